@@ -1,0 +1,62 @@
+// Internal helpers shared by the kernel sources (not part of the C ABI).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/dynaflow_hip.h"
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+#define DFHIP_DEVICE __device__ __forceinline__
+
+static inline bool dfhip_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+static inline int dfhip_check_launch() {
+  return hipGetLastError() == hipSuccess ? DFHIP_OK : DFHIP_ERR_LAUNCH;
+}
+
+// bf16 <-> fp32 on raw 16-bit storage
+DFHIP_DEVICE float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+
+// round-to-nearest-even fp32 -> bf16 (quiet NaN preserved)
+DFHIP_DEVICE uint32_t f32_to_bf16_bits(float f) {
+  bf16_t h = static_cast<bf16_t>(f);
+  return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, h));
+}
+
+DFHIP_DEVICE uint32_t pack2_bf16(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+// 64-lane reductions through DPP-free shuffles (wave64)
+DFHIP_DEVICE float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+DFHIP_DEVICE float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// The 8 XCDs of the chip take workgroups round-robin (workgroup i runs on XCD
+// i % 8) and each XCD has a private L2.  remap_xcd turns the launch index into
+// a tile index such that every XCD walks one contiguous range of tiles, so the
+// tiles that are resident together on an XCD are neighbours and share operand
+// rows/columns in that XCD's L2.
+DFHIP_DEVICE int remap_xcd(int pid, int total) {
+  constexpr int XCDS = 8;
+  const int xcd = pid % XCDS;
+  const int local = pid / XCDS;
+  const int base = total / XCDS;
+  const int rem = total % XCDS;
+  const int start = xcd * base + (xcd < rem ? xcd : rem);
+  return start + local;
+}

@@ -1,0 +1,304 @@
+"""Torch operators that front the C-ABI kernels (namespace ``dynaflow_hip``).
+
+Each operator is a ``torch.library`` definition with
+
+* a **device implementation** (dispatch key ``CUDA``, which is HIP on ROCm) that
+  passes raw device pointers and the current HIP stream to
+  ``libdynaflow_hip.so`` through ctypes, and
+* a **fake implementation** so the operators can appear inside traced FX graphs
+  (dynamo, ``fx.Interpreter`` under fake mode).
+
+There is deliberately no CPU implementation: calling one of these operators on
+host tensors, or without the built library, raises.  The operators show up in FX
+graphs as ``call_function`` nodes whose ``target.__name__`` starts with the
+operator name (``linear``, ``silu_mul``, ...), so ``matching.Op`` patterns such
+as ``r"linear(\\.default)?"`` see them like any aten function.
+
+Reference call sites these stand in for: the FX nodes ``linear``, ``silu`` and
+``mul`` of the MLP sub-graphs, executed by PyTorch at
+dynaflow/runtime/engine.py:381.
+"""
+from __future__ import annotations
+
+import torch
+
+from dynaflow_amd import _cabi
+
+_lib = torch.library.Library("dynaflow_hip", "DEF")
+
+_lib.define("linear(Tensor x, Tensor weight) -> Tensor")
+_lib.define("linear_variant(Tensor x, Tensor weight, int variant) -> Tensor")
+_lib.define("silu_mul(Tensor gate, Tensor up, bool round_silu=False) -> Tensor")
+_lib.define("rms_norm(Tensor x, Tensor weight, float eps) -> Tensor")
+_lib.define("add_rms_norm(Tensor x, Tensor residual, Tensor weight, float eps) -> (Tensor, Tensor)")
+_lib.define("transpose_weight(Tensor w) -> Tensor")
+_lib.define("quant_fp8(Tensor x) -> (Tensor, Tensor)")
+_lib.define("silu_mul_quant_fp8(Tensor gate, Tensor up) -> (Tensor, Tensor)")
+_lib.define("linear_fp8(Tensor x_q, Tensor w_q, Tensor x_scale, Tensor w_scale) -> Tensor")
+
+FP8_DTYPE = torch.float8_e4m3fn
+FP8_MAX = 448.0
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _rows(t: torch.Tensor) -> tuple[torch.Tensor, int, int, int]:
+    """View ``t[..., D]`` as rows: returns (tensor, M, D, leading dimension).
+
+    A 2-D tensor with unit stride in the last dimension is used as it is (so
+    row-strided views such as the halves of a packed gate_up buffer work);
+    anything else is flattened, copying only if it has to.
+    """
+    if t.dim() == 2 and t.stride(1) == 1 and t.stride(0) >= t.shape[1]:
+        return t, t.shape[0], t.shape[1], t.stride(0)
+    flat = t.reshape(-1, t.shape[-1])
+    if flat.stride(1) != 1 or (flat.shape[0] > 1 and flat.stride(0) < flat.shape[1]):
+        flat = flat.contiguous()
+    ld = flat.stride(0) if flat.shape[0] > 1 else flat.shape[1]
+    return flat, flat.shape[0], flat.shape[1], ld
+
+
+def _require_device(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("dynaflow_hip operators run on the GPU only; got a host tensor")
+
+
+# ---------------------------------------------------------------- linear
+def _linear_impl(x: torch.Tensor, weight: torch.Tensor, variant: int = -1) -> torch.Tensor:
+    _require_device(x, weight)
+    lib = _cabi.load()
+    if weight.dim() != 2 or x.shape[-1] != weight.shape[1]:
+        raise RuntimeError(f"linear: x[..., {x.shape[-1]}] does not match weight {tuple(weight.shape)}")
+    if x.dtype != weight.dtype:
+        raise RuntimeError(f"linear: dtype mismatch {x.dtype} vs {weight.dtype}")
+    a, M, K, lda = _rows(x)
+    w, N, _, ldw = _rows(weight)
+    out = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    if M > 0:
+        if x.dtype == torch.bfloat16:
+            if variant >= 0:
+                rc = lib.dfhip_gemm_bf16_nt_variant(
+                    a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), N, M, N, K, variant, _stream()
+                )
+                _cabi.check("dfhip_gemm_bf16_nt_variant", rc)
+            else:
+                rc = lib.dfhip_gemm_bf16_nt(
+                    a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), N, M, N, K, _stream()
+                )
+                _cabi.check("dfhip_gemm_bf16_nt", rc)
+        elif x.dtype == torch.float32:
+            rc = lib.dfhip_gemm_f32_nt(
+                a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), N, M, N, K, _stream()
+            )
+            _cabi.check("dfhip_gemm_f32_nt", rc)
+        else:
+            raise RuntimeError(f"linear: unsupported dtype {x.dtype}")
+    return out.view(*x.shape[:-1], N)
+
+
+def _linear_fake(x, weight):
+    return x.new_empty((*x.shape[:-1], weight.shape[0]))
+
+
+_lib.impl("linear", lambda x, w: _linear_impl(x, w), "CUDA")
+_lib.impl("linear_variant", lambda x, w, v: _linear_impl(x, w, v), "CUDA")
+torch.library.register_fake("dynaflow_hip::linear", _linear_fake, lib=_lib)
+torch.library.register_fake("dynaflow_hip::linear_variant", lambda x, w, v: _linear_fake(x, w), lib=_lib)
+
+
+# -------------------------------------------------------------- silu * mul
+def _silu_mul_impl(gate: torch.Tensor, up: torch.Tensor, round_silu: bool = False) -> torch.Tensor:
+    _require_device(gate, up)
+    lib = _cabi.load()
+    if gate.shape != up.shape or gate.dtype != up.dtype:
+        raise RuntimeError("silu_mul: gate and up must agree in shape and dtype")
+    g, M, D, ldg = _rows(gate)
+    u, _, _, ldu = _rows(up)
+    out = torch.empty((M, D), dtype=gate.dtype, device=gate.device)
+    if M > 0:
+        if gate.dtype == torch.bfloat16:
+            rc = lib.dfhip_silu_mul_bf16(
+                g.data_ptr(), ldg, u.data_ptr(), ldu, out.data_ptr(), D, M, D, int(round_silu), _stream()
+            )
+            _cabi.check("dfhip_silu_mul_bf16", rc)
+        elif gate.dtype == torch.float32:
+            rc = lib.dfhip_silu_mul_f32(
+                g.data_ptr(), ldg, u.data_ptr(), ldu, out.data_ptr(), D, M, D, _stream()
+            )
+            _cabi.check("dfhip_silu_mul_f32", rc)
+        else:
+            raise RuntimeError(f"silu_mul: unsupported dtype {gate.dtype}")
+    return out.view(gate.shape)
+
+
+_lib.impl("silu_mul", _silu_mul_impl, "CUDA")
+torch.library.register_fake(
+    "dynaflow_hip::silu_mul", lambda gate, up, round_silu=False: torch.empty_like(gate), lib=_lib
+)
+
+
+# ----------------------------------------------------------------- rmsnorm
+def _rms_norm_impl(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    _require_device(x, weight)
+    lib = _cabi.load()
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise RuntimeError("rms_norm: bf16 only")
+    xr = x.reshape(-1, x.shape[-1]).contiguous()
+    out = torch.empty_like(xr)
+    if xr.shape[0] > 0:
+        rc = lib.dfhip_rmsnorm_bf16(
+            xr.data_ptr(), None, weight.contiguous().data_ptr(), out.data_ptr(), None,
+            xr.shape[0], xr.shape[1], float(eps), _stream(),
+        )
+        _cabi.check("dfhip_rmsnorm_bf16", rc)
+    return out.view(x.shape)
+
+
+def _add_rms_norm_impl(x, residual, weight, eps):
+    _require_device(x, residual, weight)
+    lib = _cabi.load()
+    if x.dtype != torch.bfloat16 or residual.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise RuntimeError("add_rms_norm: bf16 only")
+    xr = x.reshape(-1, x.shape[-1]).contiguous()
+    rr = residual.reshape(-1, x.shape[-1]).contiguous()
+    out = torch.empty_like(xr)
+    res_out = torch.empty_like(xr)
+    if xr.shape[0] > 0:
+        rc = lib.dfhip_rmsnorm_bf16(
+            xr.data_ptr(), rr.data_ptr(), weight.contiguous().data_ptr(), out.data_ptr(),
+            res_out.data_ptr(), xr.shape[0], xr.shape[1], float(eps), _stream(),
+        )
+        _cabi.check("dfhip_rmsnorm_bf16", rc)
+    return out.view(x.shape), res_out.view(x.shape)
+
+
+_lib.impl("rms_norm", _rms_norm_impl, "CUDA")
+_lib.impl("add_rms_norm", _add_rms_norm_impl, "CUDA")
+torch.library.register_fake("dynaflow_hip::rms_norm", lambda x, w, eps: torch.empty_like(x), lib=_lib)
+torch.library.register_fake(
+    "dynaflow_hip::add_rms_norm", lambda x, r, w, eps: (torch.empty_like(x), torch.empty_like(x)), lib=_lib
+)
+
+
+# ------------------------------------------------------ weight re-layout
+def _transpose_weight_impl(w: torch.Tensor) -> torch.Tensor:
+    """[K, N] (``x @ W`` convention) -> [N, K] (``linear`` convention), bf16."""
+    _require_device(w)
+    lib = _cabi.load()
+    if w.dim() != 2 or w.dtype != torch.bfloat16:
+        raise RuntimeError("transpose_weight: 2-D bf16 only")
+    src, K, N, ld = _rows(w)
+    out = torch.empty((N, K), dtype=w.dtype, device=w.device)
+    rc = lib.dfhip_transpose_bf16(src.data_ptr(), ld, out.data_ptr(), K, K, N, _stream())
+    _cabi.check("dfhip_transpose_bf16", rc)
+    return out
+
+
+_lib.impl("transpose_weight", _transpose_weight_impl, "CUDA")
+torch.library.register_fake(
+    "dynaflow_hip::transpose_weight", lambda w: w.new_empty((w.shape[1], w.shape[0])), lib=_lib
+)
+
+
+# --------------------------------------------------------------------- fp8
+def _fill_zero(t: torch.Tensor) -> None:
+    rc = _cabi.load().dfhip_fill_u32(t.data_ptr(), 0, t.numel(), _stream())
+    _cabi.check("dfhip_fill_u32", rc)
+
+
+def _quant_fp8_impl(x: torch.Tensor):
+    """Per-tensor dynamic quantisation: returns (e4m3fn tensor, scale[1] fp32)."""
+    _require_device(x)
+    lib = _cabi.load()
+    if x.dtype != torch.bfloat16:
+        raise RuntimeError("quant_fp8: bf16 input only")
+    xr, M, D, ld = _rows(x)
+    amax = torch.empty(1, dtype=torch.float32, device=x.device)
+    scale = torch.empty(1, dtype=torch.float32, device=x.device)
+    q = torch.empty((M, D), dtype=FP8_DTYPE, device=x.device)
+    _fill_zero(amax)
+    rc = lib.dfhip_absmax_bf16(xr.data_ptr(), ld, M, D, amax.data_ptr(), _stream())
+    _cabi.check("dfhip_absmax_bf16", rc)
+    rc = lib.dfhip_quant_fp8_bf16(
+        xr.data_ptr(), ld, q.data_ptr(), D, M, D, amax.data_ptr(), scale.data_ptr(), _stream()
+    )
+    _cabi.check("dfhip_quant_fp8_bf16", rc)
+    return q.view(x.shape), scale
+
+
+def _silu_mul_quant_fp8_impl(gate: torch.Tensor, up: torch.Tensor):
+    """silu(gate)*up, re-quantised per tensor: returns (e4m3fn tensor, scale[1])."""
+    _require_device(gate, up)
+    lib = _cabi.load()
+    if gate.dtype != torch.bfloat16 or gate.shape != up.shape or up.dtype != torch.bfloat16:
+        raise RuntimeError("silu_mul_quant_fp8: two bf16 tensors of one shape")
+    g, M, D, ldg = _rows(gate)
+    u, _, _, ldu = _rows(up)
+    act = torch.empty((M, D), dtype=torch.bfloat16, device=gate.device)
+    amax = torch.empty(1, dtype=torch.float32, device=gate.device)
+    scale = torch.empty(1, dtype=torch.float32, device=gate.device)
+    q = torch.empty((M, D), dtype=FP8_DTYPE, device=gate.device)
+    _fill_zero(amax)
+    rc = lib.dfhip_silu_mul_absmax_bf16(
+        g.data_ptr(), ldg, u.data_ptr(), ldu, act.data_ptr(), D, M, D, amax.data_ptr(), _stream()
+    )
+    _cabi.check("dfhip_silu_mul_absmax_bf16", rc)
+    rc = lib.dfhip_quant_fp8_bf16(
+        act.data_ptr(), D, q.data_ptr(), D, M, D, amax.data_ptr(), scale.data_ptr(), _stream()
+    )
+    _cabi.check("dfhip_quant_fp8_bf16", rc)
+    return q.view(gate.shape), scale
+
+
+def _linear_fp8_impl(x_q, w_q, x_scale, w_scale):
+    _require_device(x_q, w_q, x_scale, w_scale)
+    lib = _cabi.load()
+    if x_q.dtype != FP8_DTYPE or w_q.dtype != FP8_DTYPE:
+        raise RuntimeError("linear_fp8: e4m3fn operands only")
+    if x_scale.dtype != torch.float32 or w_scale.dtype != torch.float32:
+        raise RuntimeError("linear_fp8: fp32 scales only")
+    a, M, K, lda = _rows(x_q)
+    w, N, Kw, ldw = _rows(w_q)
+    if K != Kw or w_scale.numel() != N or x_scale.numel() != 1:
+        raise RuntimeError("linear_fp8: shape mismatch")
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=x_q.device)
+    if M > 0:
+        rc = lib.dfhip_gemm_fp8_nt(
+            a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), N,
+            x_scale.data_ptr(), w_scale.contiguous().data_ptr(), M, N, K, _stream(),
+        )
+        _cabi.check("dfhip_gemm_fp8_nt", rc)
+    return out.view(*x_q.shape[:-1], N)
+
+
+_lib.impl("quant_fp8", _quant_fp8_impl, "CUDA")
+_lib.impl("silu_mul_quant_fp8", _silu_mul_quant_fp8_impl, "CUDA")
+_lib.impl("linear_fp8", _linear_fp8_impl, "CUDA")
+torch.library.register_fake(
+    "dynaflow_hip::quant_fp8",
+    lambda x: (x.new_empty(x.shape, dtype=FP8_DTYPE), x.new_empty((1,), dtype=torch.float32)),
+    lib=_lib,
+)
+torch.library.register_fake(
+    "dynaflow_hip::silu_mul_quant_fp8",
+    lambda g, u: (g.new_empty(g.shape, dtype=FP8_DTYPE), g.new_empty((1,), dtype=torch.float32)),
+    lib=_lib,
+)
+torch.library.register_fake(
+    "dynaflow_hip::linear_fp8",
+    lambda x_q, w_q, xs, ws: x_q.new_empty((*x_q.shape[:-1], w_q.shape[0]), dtype=torch.bfloat16),
+    lib=_lib,
+)
+
+linear = torch.ops.dynaflow_hip.linear
+linear_variant = torch.ops.dynaflow_hip.linear_variant
+silu_mul = torch.ops.dynaflow_hip.silu_mul
+rms_norm = torch.ops.dynaflow_hip.rms_norm
+add_rms_norm = torch.ops.dynaflow_hip.add_rms_norm
+transpose_weight = torch.ops.dynaflow_hip.transpose_weight
+quant_fp8 = torch.ops.dynaflow_hip.quant_fp8
+silu_mul_quant_fp8 = torch.ops.dynaflow_hip.silu_mul_quant_fp8
+linear_fp8 = torch.ops.dynaflow_hip.linear_fp8

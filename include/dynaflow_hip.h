@@ -1,0 +1,158 @@
+/*
+ * dynaflow_hip.h - C ABI of the MI355X (gfx950) kernel library behind the
+ * DynaFlow scheduling layer.
+ *
+ * The reference has no kernel library of its own: its sub-graphs run whatever
+ * PyTorch dispatches for their FX nodes (dynaflow/runtime/engine.py:160,220,
+ * 325,381,491), optionally compiled by TorchInductor
+ * (dynaflow/executor/inductor.py:111-141).  This library takes that slot for
+ * the batch-split SwiGLU MLP path.  Each entry point below names the
+ * reference call site or kernel whose arithmetic it replaces.
+ *
+ * Conventions (all entry points):
+ *   - plain pointers and sizes, no framework types; pointers are device
+ *     pointers unless stated otherwise;
+ *   - the HIP stream is passed explicitly (NULL = the null stream);
+ *   - nothing allocates, frees or synchronises; every call is legal under
+ *     stream capture;
+ *   - the return value is DFHIP_OK (0) or a negative dfhip_status; shapes,
+ *     strides and alignment are checked before anything is launched;
+ *   - row-major matrices with leading dimensions given in ELEMENTS;
+ *   - bf16 values are the upper 16 bits of an IEEE fp32 (uint16_t storage),
+ *     fp8 values are OCP e4m3fn (uint8_t storage).
+ */
+#ifndef DYNAFLOW_HIP_H
+#define DYNAFLOW_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* dfhip_stream_t; /* hipStream_t */
+
+typedef enum dfhip_status {
+  DFHIP_OK = 0,
+  DFHIP_ERR_NULL_POINTER = -1,
+  DFHIP_ERR_BAD_SHAPE = -2,     /* non-positive or unsupported extents */
+  DFHIP_ERR_BAD_STRIDE = -3,    /* leading dimension smaller than the row */
+  DFHIP_ERR_BAD_ALIGNMENT = -4, /* pointer or stride not 16-byte aligned */
+  DFHIP_ERR_LAUNCH = -5,        /* hipGetLastError() after the launch */
+  DFHIP_ERR_NO_DEVICE = -6,
+  DFHIP_ERR_BAD_ARGUMENT = -7
+} dfhip_status;
+
+typedef struct dfhip_device_info {
+  int compute_units;
+  int clock_khz;           /* peak engine clock */
+  int memory_clock_khz;
+  int memory_bus_bits;
+  int lds_bytes_per_block; /* max opt-in LDS per workgroup */
+  int wavefront_size;
+  char arch_name[64];      /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+} dfhip_device_info;
+
+/* Library ABI version (major*1000 + minor). */
+int dfhip_version(void);
+/* The architecture the device code was compiled for ("gfx950"). */
+const char* dfhip_arch(void);
+/* Text for a dfhip_status. */
+const char* dfhip_status_string(int status);
+/* Properties of `device` (host struct).  Counterpart of the cached
+ * attribute helpers in
+ * examples/ae/scheduler/vllm/tokenweave-kernels/csrc/cuda_utils.cu:3-26. */
+int dfhip_device_info_get(int device, dfhip_device_info* out);
+
+/* ------------------------------------------------------------------ GEMMs
+ *
+ * C[M,N] = A[M,K] * W[N,K]^T  - the `linear` FX node of the sub-graphs
+ * (torch.nn.functional.linear, weight stored [out_features, in_features];
+ * launched at dynaflow/runtime/engine.py:381).  fp32 accumulation.
+ *
+ * bf16: A, W, C are bf16.  Requires K % 64 == 0, N % 8 == 0, lda/ldw/ldc % 8
+ * == 0 and 16-byte aligned pointers.  Any M >= 1.
+ */
+int dfhip_gemm_bf16_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                       int64_t ldc, int M, int N, int K, dfhip_stream_t stream);
+
+/* Same contraction with an explicit kernel variant, for tuning and tests.
+ * variant: 0 = 256x256 tile / 4 waves, 1 = 256x256 / 8 waves,
+ *          2 = 128x128 / 4 waves, 3 = 256x128 / 4 waves. */
+int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                               int64_t ldc, int M, int N, int K, int variant,
+                               dfhip_stream_t stream);
+
+/* fp32 in / fp32 accumulate / fp32 out (the CPU-sized fp32 configuration).
+ * Requires K % 4 == 0, 16-byte aligned pointers, lda/ldw % 4 == 0. */
+int dfhip_gemm_f32_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                      int64_t ldc, int M, int N, int K, dfhip_stream_t stream);
+
+/* fp8 e4m3fn inputs, fp32 accumulate, bf16 output:
+ *   C[m,n] = bf16( a_scale[0] * w_scale[n] * sum_k A[m,k] * W[n,k] )
+ * a_scale: device pointer to ONE float (per-tensor dynamic scale),
+ * w_scale: device pointer to N floats (per-output-channel scale).
+ * Requires K % 128 == 0, N % 8 == 0, lda/ldw % 16 == 0, ldc % 8 == 0. */
+int dfhip_gemm_fp8_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                      int64_t ldc, const float* a_scale, const float* w_scale, int M, int N,
+                      int K, dfhip_stream_t stream);
+
+/* ------------------------------------------------------------ elementwise
+ *
+ * out[t,j] = bf16( (g / (1 + expf(-g))) * u ),  g = gate[t,j], u = up[t,j],
+ * fp32 arithmetic, one rounding at the store - the `silu` and `mul` FX nodes,
+ * written out in examples/ae/up-silu-overlap.cu:75-90.  `gate` and `up` have
+ * their own row strides, so a packed gate_up[M, 2D] buffer is passed as
+ * (gate = buf, up = buf + D, ld = 2D).  Requires D % 8 == 0, strides % 8 == 0.
+ * With round_inputs_product != 0 the value silu(g) is first rounded to bf16
+ * and then multiplied (what two separate bf16 aten kernels produce). */
+int dfhip_silu_mul_bf16(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                        void* out, int64_t ld_out, int M, int D, int round_inputs_product,
+                        dfhip_stream_t stream);
+
+/* fp32 flavour of the same op (fp32 configuration). D % 4 == 0. */
+int dfhip_silu_mul_f32(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                       void* out, int64_t ld_out, int M, int D, dfhip_stream_t stream);
+
+/* RMSNorm over rows of x[M,H] (bf16), optional residual add:
+ *   h = bf16(x + residual)            (residual may be NULL; written back to
+ *                                      `residual_out` when that is not NULL)
+ *   out = bf16( bf16(h * rsqrtf(mean(h^2) + eps)) * weight )
+ * fp32 sum of squares; the arithmetic of
+ * examples/ae/scheduler/vllm/tokenweave-kernels/csrc/tokenweave.cu:85-109
+ * without its cross-GPU parts.  Requires H % 8 == 0 and H <= 16384. */
+int dfhip_rmsnorm_bf16(const void* x, const void* residual, const void* weight, void* out,
+                       void* residual_out, int M, int H, float eps, dfhip_stream_t stream);
+
+/* out[N,K] = in[K,N]^T for bf16 matrices: packs a weight kept as [in, out]
+ * (x @ W convention) into the [out, in] layout the GEMMs read.  K, N % 8 == 0. */
+int dfhip_transpose_bf16(const void* in, int64_t ld_in, void* out, int64_t ld_out, int K, int N,
+                         dfhip_stream_t stream);
+
+/* ------------------------------------------------------------------- fp8
+ *
+ * Per-tensor dynamic quantisation of a bf16 activation to e4m3fn in two
+ * launches: (1) amax[0] = max |x| (fp32; the caller zero-fills amax[0] before
+ * the launch), (2) scale[0] = max(amax, 1e-12) / 448, q = e4m3fn(x / scale[0]),
+ * round-to-nearest-even, saturating at +-448. */
+int dfhip_absmax_bf16(const void* x, int64_t ld, int M, int D, float* amax,
+                      dfhip_stream_t stream);
+int dfhip_quant_fp8_bf16(const void* x, int64_t ld, void* q, int64_t ld_q, int M, int D,
+                         const float* amax, float* scale_out, dfhip_stream_t stream);
+
+/* silu(gate)*up in fp32 from bf16 inputs, written as bf16 to `out` (may be
+ * NULL) and reduced into amax[0] = max |silu(g)*u| for the following
+ * re-quantisation of the down-projection's input. */
+int dfhip_silu_mul_absmax_bf16(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                               void* out, int64_t ld_out, int M, int D, float* amax,
+                               dfhip_stream_t stream);
+
+/* Fill `count` 32-bit words with `value` (a capture-safe replacement for
+ * memset nodes, used to clear amax cells). */
+int dfhip_fill_u32(void* dst, uint32_t value, int64_t count, dfhip_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DYNAFLOW_HIP_H */
