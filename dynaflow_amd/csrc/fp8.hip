@@ -1,0 +1,322 @@
+// fp8 (OCP e4m3fn) path: per-tensor dynamic quantisation, SiLU*mul with amax,
+// and the fp8 GEMM  C = bf16(a_scale * w_scale[n] * A[M,K] * W[N,K]^T).
+//
+// The GEMM has the byte geometry of the bf16 one (a K slab row is 128 bytes,
+// here 128 fp8 values): 16-byte global loads staged through registers into two
+// padded LDS buffers, one barrier per slab.  It multiplies with
+// v_mfma_scale_f32_32x32x64_f8f6f4 (scale exponents fixed at 2^0), which
+// retires 64 k per instruction - twice the bf16 rate.  A lane feeds 32
+// consecutive bytes of one row; both operands use the same lane->k mapping, so
+// the contraction is exact whatever order the hardware walks those bytes in.
+#include "dfhip_common.h"
+
+namespace {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+constexpr float FP8_MAX = 448.0f;
+constexpr int QT = 256;      // threads of the elementwise fp8 kernels
+constexpr int QUNROLL = 4;
+
+DFHIP_DEVICE float silu_f32(float g) { return g / (1.0f + expf(-g)); }
+
+DFHIP_DEVICE void atomic_max_nonneg(float* cell, float v) {
+  // non-negative floats order like their bit patterns
+  atomicMax(reinterpret_cast<unsigned int*>(cell), __float_as_uint(v));
+}
+
+DFHIP_DEVICE void block_max_to(float* cell, float v) {
+  __shared__ float partial[QT / 64];
+  v = wave_max(v);
+  if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = v;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float m = partial[0];
+#pragma unroll
+    for (int w = 1; w < QT / 64; ++w) m = fmaxf(m, partial[w]);
+    atomic_max_nonneg(cell, m);
+  }
+}
+
+// amax[0] = max(amax[0], max |x|) over a row-strided bf16 matrix; group = 8 values
+__global__ void __launch_bounds__(QT)
+absmax_bf16_kernel(const uint16_t* __restrict__ x, int64_t ld, uint32_t groups, uint32_t per_row,
+                   float* __restrict__ amax) {
+  float m = 0.0f;
+  for (uint32_t gi = blockIdx.x * QT + threadIdx.x; gi < groups; gi += gridDim.x * QT) {
+    const uint32_t row = gi / per_row, col = (gi - row * per_row) * 8;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(x + (int64_t)row * ld + col);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      m = fmaxf(m, fabsf(bf16_bits_to_f32(v[w] & 0xffffu)));
+      m = fmaxf(m, fabsf(__uint_as_float(v[w] & 0xffff0000u)));
+    }
+  }
+  block_max_to(amax, m);
+}
+
+DFHIP_DEVICE uint32_t quant4(float a, float b, float c, float d, float scale) {
+  a = fminf(fmaxf(a / scale, -FP8_MAX), FP8_MAX);
+  b = fminf(fmaxf(b / scale, -FP8_MAX), FP8_MAX);
+  c = fminf(fmaxf(c / scale, -FP8_MAX), FP8_MAX);
+  d = fminf(fmaxf(d / scale, -FP8_MAX), FP8_MAX);
+  uint32_t r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);  // bytes 0,1
+  r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);            // bytes 2,3
+  return r;
+}
+
+// q = e4m3fn(x / scale), scale = max(amax, 1e-12) / 448; group = 8 values -> 8 bytes
+__global__ void __launch_bounds__(QT)
+quant_fp8_bf16_kernel(const uint16_t* __restrict__ x, int64_t ld, uint8_t* __restrict__ q, int64_t ld_q,
+                      uint32_t groups, uint32_t per_row, const float* __restrict__ amax,
+                      float* __restrict__ scale_out) {
+  const float scale = fmaxf(amax[0], 1e-12f) / FP8_MAX;
+  if (blockIdx.x == 0 && threadIdx.x == 0 && scale_out != nullptr) scale_out[0] = scale;
+  for (uint32_t gi = blockIdx.x * QT + threadIdx.x; gi < groups; gi += gridDim.x * QT) {
+    const uint32_t row = gi / per_row, col = (gi - row * per_row) * 8;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(x + (int64_t)row * ld + col);
+    u32x2 o;
+    o[0] = quant4(bf16_bits_to_f32(v[0] & 0xffffu), __uint_as_float(v[0] & 0xffff0000u),
+                  bf16_bits_to_f32(v[1] & 0xffffu), __uint_as_float(v[1] & 0xffff0000u), scale);
+    o[1] = quant4(bf16_bits_to_f32(v[2] & 0xffffu), __uint_as_float(v[2] & 0xffff0000u),
+                  bf16_bits_to_f32(v[3] & 0xffffu), __uint_as_float(v[3] & 0xffff0000u), scale);
+    *reinterpret_cast<u32x2*>(q + (int64_t)row * ld_q + col) = o;
+  }
+}
+
+// out = bf16(silu(g) * u) (optional store) and amax over the rounded values
+__global__ void __launch_bounds__(QT)
+silu_mul_absmax_kernel(const uint16_t* __restrict__ gate, int64_t ld_gate, const uint16_t* __restrict__ up,
+                       int64_t ld_up, uint16_t* __restrict__ out, int64_t ld_out, uint32_t groups,
+                       uint32_t per_row, float* __restrict__ amax) {
+  float m = 0.0f;
+  for (uint32_t gi = blockIdx.x * QT + threadIdx.x; gi < groups; gi += gridDim.x * QT) {
+    const uint32_t row = gi / per_row, col = (gi - row * per_row) * 8;
+    const u32x4 g = *reinterpret_cast<const u32x4*>(gate + (int64_t)row * ld_gate + col);
+    const u32x4 u = *reinterpret_cast<const u32x4*>(up + (int64_t)row * ld_up + col);
+    u32x4 o;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float lo = silu_f32(bf16_bits_to_f32(g[w] & 0xffffu)) * bf16_bits_to_f32(u[w] & 0xffffu);
+      const float hi = silu_f32(__uint_as_float(g[w] & 0xffff0000u)) * __uint_as_float(u[w] & 0xffff0000u);
+      o[w] = pack2_bf16(lo, hi);
+      m = fmaxf(m, fabsf(bf16_bits_to_f32(o[w] & 0xffffu)));
+      m = fmaxf(m, fabsf(__uint_as_float(o[w] & 0xffff0000u)));
+    }
+    if (out != nullptr) *reinterpret_cast<u32x4*>(out + (int64_t)row * ld_out + col) = o;
+  }
+  block_max_to(amax, m);
+}
+
+// ------------------------------------------------------------------ fp8 GEMM
+constexpr int FBK = 128;            // fp8 values (= bytes) per slab row
+constexpr int FROW = FBK + 16;      // padded LDS row in bytes
+constexpr int FCHUNKS = FBK / 16;   // 16-byte chunks per slab row
+
+template <int BM, int BN>
+__global__ void __launch_bounds__(256)
+gemm_fp8_nt_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, uint16_t* __restrict__ C,
+                   const float* __restrict__ a_scale, const float* __restrict__ w_scale, int M, int N, int K,
+                   int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n) {
+  constexpr int THREADS = 256;
+  constexpr int WTM = BM / 2, WTN = BN / 2, TM = WTM / 32, TN = WTN / 32;
+  constexpr int A_LOADS = BM * FCHUNKS / THREADS, W_LOADS = BN * FCHUNKS / THREADS;
+  constexpr int ROWS_PER_PASS = THREADS / FCHUNKS;
+  constexpr int BUF_BYTES = (BM + BN) * FROW;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wave_m = wave & 1, wave_n = wave >> 1;
+  const int tile = remap_xcd(blockIdx.x, tiles_m * tiles_n);
+  const int m0 = (tile % tiles_m) * BM, n0 = (tile / tiles_m) * BN;
+
+  const int ld_row = tid / FCHUNKS, ld_chunk = tid % FCHUNKS;
+  const uint8_t* a_src[A_LOADS];
+  const uint8_t* w_src[W_LOADS];
+#pragma unroll
+  for (int p = 0; p < A_LOADS; ++p) {
+    int row = m0 + ld_row + p * ROWS_PER_PASS;
+    row = row < M ? row : M - 1;
+    a_src[p] = A + (int64_t)row * lda + ld_chunk * 16;
+  }
+#pragma unroll
+  for (int p = 0; p < W_LOADS; ++p) {
+    int row = n0 + ld_row + p * ROWS_PER_PASS;
+    row = row < N ? row : N - 1;
+    w_src[p] = W + (int64_t)row * ldw + ld_chunk * 16;
+  }
+  u32x4 a_reg[A_LOADS], w_reg[W_LOADS];
+  auto fetch = [&](int kt) {
+#pragma unroll
+    for (int p = 0; p < A_LOADS; ++p) a_reg[p] = *reinterpret_cast<const u32x4*>(a_src[p] + kt * FBK);
+#pragma unroll
+    for (int p = 0; p < W_LOADS; ++p) w_reg[p] = *reinterpret_cast<const u32x4*>(w_src[p] + kt * FBK);
+  };
+  auto park = [&](int buf) {
+    uint8_t* a_dst = smem + buf * BUF_BYTES + ld_row * FROW + ld_chunk * 16;
+    uint8_t* w_dst = a_dst + BM * FROW;
+#pragma unroll
+    for (int p = 0; p < A_LOADS; ++p) *reinterpret_cast<u32x4*>(a_dst + p * ROWS_PER_PASS * FROW) = a_reg[p];
+#pragma unroll
+    for (int p = 0; p < W_LOADS; ++p) *reinterpret_cast<u32x4*>(w_dst + p * ROWS_PER_PASS * FROW) = w_reg[p];
+  };
+
+  // lane reads 32 consecutive bytes: row lane%32, byte offset 64*ks + 32*(lane/32)
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  const int a_frag_off = (wave_m * WTM + frag_row) * FROW + frag_half * 32;
+  const int w_frag_off = BM * FROW + (wave_n * WTN + frag_row) * FROW + frag_half * 32;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int KT = K / FBK;
+  fetch(0);
+  park(0);
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT) fetch(kt + 1);
+    const uint8_t* base = smem + buf * BUF_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < FBK / 64; ++ks) {
+      i32x8 fa[TM], fw[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(base + a_frag_off + i * 32 * FROW + ks * 64);
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(base + a_frag_off + i * 32 * FROW + ks * 64 + 16);
+        fa[i] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const u32x4 lo = *reinterpret_cast<const u32x4*>(base + w_frag_off + j * 32 * FROW + ks * 64);
+        const u32x4 hi = *reinterpret_cast<const u32x4*>(base + w_frag_off + j * 32 * FROW + ks * 64 + 16);
+        fw[j] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fw[j], fa[i], acc[i][j], 0, 0, 0, 0x7f7f7f7f,
+                                                                     0, 0x7f7f7f7f);
+    }
+    if (kt + 1 < KT) park(buf ^ 1);
+    __syncthreads();
+  }
+
+  // W was the first operand: lane holds row m = lane%32, columns 8g + 4*(lane/32) + 0..3
+  const float sa = a_scale[0];
+  const int m_lane = m0 + wave_m * WTM + frag_row;
+  const int n_lane = n0 + wave_n * WTN + frag_half * 4;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m_lane + i * 32;
+    if (m >= M) continue;
+    uint16_t* c_row = C + (int64_t)m * ldc;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n_lane + j * 32 + g * 8;
+        if (n < N) {
+          const f32x4 ws = *reinterpret_cast<const f32x4*>(w_scale + n);
+          u32x2 v;
+          v[0] = pack2_bf16(acc[i][j][4 * g + 0] * (sa * ws[0]), acc[i][j][4 * g + 1] * (sa * ws[1]));
+          v[1] = pack2_bf16(acc[i][j][4 * g + 2] * (sa * ws[2]), acc[i][j][4 * g + 3] * (sa * ws[3]));
+          *reinterpret_cast<u32x2*>(c_row + n) = v;
+        }
+      }
+  }
+}
+
+template <int BM, int BN>
+int launch_fp8(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, const float* a_scale,
+               const float* w_scale, int M, int N, int K, hipStream_t stream) {
+  constexpr int LDS_BYTES = 2 * (BM + BN) * FROW;
+  auto kernel = gemm_fp8_nt_kernel<BM, BN>;
+  static bool lds_opted_in = false;
+  if (!lds_opted_in) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            LDS_BYTES) != hipSuccess)
+      return DFHIP_ERR_LAUNCH;
+    lds_opted_in = true;
+  }
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(256), LDS_BYTES, stream, static_cast<const uint8_t*>(A),
+                     static_cast<const uint8_t*>(W), static_cast<uint16_t*>(C), a_scale, w_scale, M, N, K, lda, ldw,
+                     ldc, tiles_m, tiles_n);
+  return dfhip_check_launch();
+}
+
+int check_q(const void* x, int64_t ld, int M, int D) {
+  if (!x) return DFHIP_ERR_NULL_POINTER;
+  if (M < 1 || D < 8 || D % 8 != 0 || (int64_t)M * (D / 8) >= (int64_t)1 << 31) return DFHIP_ERR_BAD_SHAPE;
+  if (ld < D) return DFHIP_ERR_BAD_STRIDE;
+  if (ld % 8 || !dfhip_aligned16(x)) return DFHIP_ERR_BAD_ALIGNMENT;
+  return DFHIP_OK;
+}
+
+unsigned grid_for(uint32_t groups) {
+  uint32_t blocks = (groups + QT * QUNROLL - 1) / (QT * QUNROLL);
+  return blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
+}
+
+}  // namespace
+
+extern "C" int dfhip_absmax_bf16(const void* x, int64_t ld, int M, int D, float* amax, dfhip_stream_t stream) {
+  if (int rc = check_q(x, ld, M, D)) return rc;
+  if (!amax) return DFHIP_ERR_NULL_POINTER;
+  const uint32_t per_row = D / 8, groups = (uint32_t)M * per_row;
+  hipLaunchKernelGGL(absmax_bf16_kernel, dim3(grid_for(groups)), dim3(QT), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(x), ld, groups, per_row, amax);
+  return dfhip_check_launch();
+}
+
+extern "C" int dfhip_quant_fp8_bf16(const void* x, int64_t ld, void* q, int64_t ld_q, int M, int D,
+                                    const float* amax, float* scale_out, dfhip_stream_t stream) {
+  if (int rc = check_q(x, ld, M, D)) return rc;
+  if (!q || !amax) return DFHIP_ERR_NULL_POINTER;
+  if (ld_q < D) return DFHIP_ERR_BAD_STRIDE;
+  if (ld_q % 8 || (reinterpret_cast<uintptr_t>(q) & 7u)) return DFHIP_ERR_BAD_ALIGNMENT;
+  const uint32_t per_row = D / 8, groups = (uint32_t)M * per_row;
+  hipLaunchKernelGGL(quant_fp8_bf16_kernel, dim3(grid_for(groups)), dim3(QT), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(x), ld, static_cast<uint8_t*>(q), ld_q, groups, per_row, amax,
+                     scale_out);
+  return dfhip_check_launch();
+}
+
+extern "C" int dfhip_silu_mul_absmax_bf16(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+                                          void* out, int64_t ld_out, int M, int D, float* amax,
+                                          dfhip_stream_t stream) {
+  if (int rc = check_q(gate, ld_gate, M, D)) return rc;
+  if (int rc = check_q(up, ld_up, M, D)) return rc;
+  if (!amax) return DFHIP_ERR_NULL_POINTER;
+  if (out) {
+    if (ld_out < D) return DFHIP_ERR_BAD_STRIDE;
+    if (ld_out % 8 || !dfhip_aligned16(out)) return DFHIP_ERR_BAD_ALIGNMENT;
+  }
+  const uint32_t per_row = D / 8, groups = (uint32_t)M * per_row;
+  hipLaunchKernelGGL(silu_mul_absmax_kernel, dim3(grid_for(groups)), dim3(QT), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(gate), ld_gate, static_cast<const uint16_t*>(up), ld_up,
+                     static_cast<uint16_t*>(out), ld_out, groups, per_row, amax);
+  return dfhip_check_launch();
+}
+
+extern "C" int dfhip_gemm_fp8_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
+                                 const float* a_scale, const float* w_scale, int M, int N, int K,
+                                 dfhip_stream_t stream) {
+  if (!A || !W || !C || !a_scale || !w_scale) return DFHIP_ERR_NULL_POINTER;
+  if (M < 1 || N < 1 || K < 1 || K % FBK != 0 || N % 8 != 0) return DFHIP_ERR_BAD_SHAPE;
+  if (lda < K || ldw < K || ldc < N) return DFHIP_ERR_BAD_STRIDE;
+  if (lda % 16 || ldw % 16 || ldc % 8 || !dfhip_aligned16(A) || !dfhip_aligned16(W) || !dfhip_aligned16(C) ||
+      !dfhip_aligned16(w_scale))
+    return DFHIP_ERR_BAD_ALIGNMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+  if (M > 128 && big_tiles >= 192) return launch_fp8<256, 256>(A, lda, W, ldw, C, ldc, a_scale, w_scale, M, N, K, s);
+  return launch_fp8<128, 128>(A, lda, W, ldw, C, ldc, a_scale, w_scale, M, N, K, s);
+}

@@ -1,0 +1,130 @@
+"""Rewrite a traced sub-graph onto the hand-written HIP operators.
+
+This pass takes the slot that TorchInductor has in the reference
+(dynaflow/executor/inductor.py:111-141 compiles a deep copy of the sub-graph):
+it deep-copies the sub-``GraphModule`` and replaces
+
+* ``linear(x, w)`` (no bias, bf16 or fp32)            -> ``dynaflow_hip.linear``
+* ``mul(silu(g), u)`` / ``mul(u, silu(g))``           -> ``dynaflow_hip.silu_mul``
+
+Everything else stays as traced and keeps running on PyTorch's own ROCm
+kernels.  The pass only decides by what tracing recorded (``example_value``
+dtypes and static trailing dimensions); token counts stay symbolic.
+
+``silu_mul`` is emitted with ``round_silu=True`` for bf16: two separate bf16
+aten kernels round ``silu(g)`` to bf16 before the product, and so does this.
+"""
+from __future__ import annotations
+
+import copy
+import operator
+from typing import Any
+
+import torch
+import torch.fx as fx
+
+_LINEAR_NAMES = {"linear"}
+_SILU_NAMES = {"silu"}
+_MUL_TARGETS = {operator.mul, torch.mul}
+
+
+def _target_name(node: fx.Node) -> str | None:
+    if node.op != "call_function":
+        return None
+    return getattr(node.target, "__name__", None)
+
+
+def _example(node: Any) -> Any:
+    if isinstance(node, fx.Node):
+        return node.meta.get("example_value", None)
+    return None
+
+
+def _static_int(value: Any) -> int | None:
+    return value if isinstance(value, int) and not isinstance(value, torch.SymInt) else None
+
+
+def _linear_supported(x: Any, w: Any) -> bool:
+    ex, ew = _example(x), _example(w)
+    if not isinstance(ex, torch.Tensor) or not isinstance(ew, torch.Tensor):
+        return False
+    if ex.dtype != ew.dtype or ew.dim() != 2 or ex.dim() < 2:
+        return False
+    n, k = _static_int(ew.shape[0]), _static_int(ew.shape[1])
+    if n is None or k is None:
+        return False
+    if ex.dtype == torch.bfloat16:
+        return k % 64 == 0 and n % 8 == 0
+    if ex.dtype == torch.float32:
+        return k % 4 == 0
+    return False
+
+
+def _silu_mul_supported(g: Any) -> bool:
+    eg = _example(g)
+    if not isinstance(eg, torch.Tensor) or eg.dim() < 1:
+        return False
+    d = _static_int(eg.shape[-1])
+    if d is None:
+        return False
+    if eg.dtype == torch.bfloat16:
+        return d % 8 == 0
+    if eg.dtype == torch.float32:
+        return d % 4 == 0
+    return False
+
+
+def lower_to_hip(gm: fx.GraphModule) -> tuple[fx.GraphModule, dict[str, int]]:
+    """Return a lowered deep copy of ``gm`` and a count of each rewrite."""
+    # registering the operators is a side effect of importing them
+    from dynaflow_amd import ops
+
+    lowered = copy.deepcopy(gm)
+    graph = lowered.graph
+    stats = {"linear": 0, "silu_mul": 0}
+
+    for node in list(graph.nodes):
+        name = _target_name(node)
+        if name in _LINEAR_NAMES and node.target is not ops.linear:
+            bias = node.args[2] if len(node.args) > 2 else node.kwargs.get("bias", None)
+            if bias is not None or len(node.args) < 2:
+                continue
+            x, w = node.args[0], node.args[1]
+            if not _linear_supported(x, w):
+                continue
+            with graph.inserting_before(node):
+                new = graph.call_function(ops.linear, (x, w))
+            new.meta = dict(node.meta)
+            node.replace_all_uses_with(new)
+            graph.erase_node(node)
+            stats["linear"] += 1
+
+    for node in list(graph.nodes):
+        if node.op != "call_function" or node.target not in _MUL_TARGETS or len(node.args) != 2:
+            continue
+        lhs, rhs = node.args
+        for silu, other in ((lhs, rhs), (rhs, lhs)):
+            if not isinstance(silu, fx.Node) or not isinstance(other, fx.Node):
+                continue
+            if _target_name(silu) not in _SILU_NAMES or len(silu.users) != 1:
+                continue
+            if silu.kwargs.get("inplace", False):
+                continue
+            gate = silu.args[0]
+            eg, eo = _example(gate), _example(other)
+            if not _silu_mul_supported(gate) or not isinstance(eo, torch.Tensor):
+                continue
+            if eg.dtype != eo.dtype or eg.dim() != eo.dim():
+                continue
+            with graph.inserting_before(node):
+                new = graph.call_function(ops.silu_mul, (gate, other, eg.dtype == torch.bfloat16))
+            new.meta = dict(node.meta)
+            node.replace_all_uses_with(new)
+            graph.erase_node(node)
+            graph.erase_node(silu)
+            stats["silu_mul"] += 1
+            break
+
+    graph.lint()
+    lowered.recompile()
+    return lowered, stats

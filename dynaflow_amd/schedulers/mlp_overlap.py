@@ -1,0 +1,79 @@
+"""Scheduler for the batch-split SwiGLU MLP: GEMM beside SiLU*mul + down-proj.
+
+The graph ``g = gate(x); u = up(x); y = down(silu(g) * u)`` is cut in front of
+``silu`` so that every nano-batch consists of two sub-graphs:
+
+    submod_0  gate and up projection          (no tag)         -> stream "main"
+    submod_1  SiLU*mul and down projection    (tag "tail")     -> stream "side"
+
+and the staggered order of ``StaggeredScheduler`` issues
+``(s0,b0) (s1,b0) (s0,b1) (s1,b1) ...``: nano-batch i+1's gate/up GEMM runs
+beside nano-batch i's SiLU*mul and down projection.  ``schedule="round_robin"``
+selects the NanoFlow order instead; both give the same per-stream order.
+
+Split policy: ``additional_config["num_nano_batches"]`` equal chunks (default
+``max_num_splits``); with ``split_policy="balanced"`` the two-way balanced cut
+at a request boundary.
+"""
+from __future__ import annotations
+
+from dynaflow_amd.config import DynaFlowConfig
+from dynaflow_amd.interface import ExecutionContext, InputInfo, SplitConfig
+from dynaflow_amd.matching import MatchingRule, Op
+from dynaflow_amd.schedulers.nanoflow import NanoFlowScheduler
+from dynaflow_amd.schedulers.policies import balanced_two_way, equal_n_way
+from dynaflow_amd.schedulers.staggered import StaggeredScheduler
+
+_LINEAR = r"linear(\.default)?"
+_SILU = r"silu(\.default)?"
+_MUL = r"mul(\.Tensor)?"
+
+TAIL_TAG = "tail"
+
+
+def mlp_split_rules() -> list[MatchingRule]:
+    return [
+        # silu -> mul -> down projection traced back to back
+        MatchingRule(condition=(Op(_SILU), Op(_MUL), Op(_LINEAR))),
+        # silu traced between the two projections: cut at the product instead
+        MatchingRule(condition=(Op(_MUL), Op(_LINEAR))),
+        # already fused elementwise operator
+        MatchingRule(condition=(Op(r"silu_mul(\.default)?"), Op(_LINEAR))),
+        # fp8 block: SiLU*mul + re-quantisation, then the fp8 down projection
+        MatchingRule(condition=(Op(r"silu_mul_quant_fp8(\.default)?"), Op(r"linear_fp8(\.default)?"))),
+    ]
+
+
+def mlp_tag_rules() -> dict[MatchingRule, set[str]]:
+    return {
+        MatchingRule(condition=Op(_MUL)): {TAIL_TAG},
+        MatchingRule(condition=Op(r"silu_mul(\.default)?")): {TAIL_TAG},
+        MatchingRule(condition=Op(r"silu_mul_quant_fp8(\.default)?")): {TAIL_TAG},
+    }
+
+
+class MLPOverlapScheduler(StaggeredScheduler):
+    def __init__(self, config: DynaFlowConfig) -> None:
+        super().__init__(config, mlp_split_rules(), mlp_tag_rules(), side_tag=TAIL_TAG)
+        self.policy_name = "mlp_overlap"
+        self.num_nano_batches = config.knob("num_nano_batches", config.max_num_splits)
+        self.split_policy = config.knob("split_policy", "equal")
+        self.order = config.knob("schedule", "staggered")
+        self.capture_sizes = config.cudagraph_config.capture_sizes
+        self.serialize = bool(config.knob("serialize", False))
+        if self.serialize:
+            # debugging / baseline mode: every launch on one stream
+            self.comm_stream = self.comp_stream
+
+    def get_split_config(self, input_info: InputInfo, use_cudagraph: bool = False) -> SplitConfig:
+        if self.split_policy == "balanced":
+            return balanced_two_way(
+                input_info, use_cudagraph, self.min_nano_split_tokens, self.capture_sizes or [0]
+            )
+        return equal_n_way(input_info, use_cudagraph, self.num_nano_batches, self.min_nano_split_tokens)
+
+    async def schedule(self, context: ExecutionContext) -> None:
+        if self.order == "round_robin":
+            await NanoFlowScheduler.schedule(self, context)  # type: ignore[arg-type]
+        else:
+            await super().schedule(context)

@@ -1,0 +1,71 @@
+"""The C-ABI library loads on a host without a GPU and exports every symbol that
+include/dynaflow_hip.h declares (no kernel is launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from dynaflow_amd import _cabi
+
+HEADER = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "dynaflow_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dfhip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert declared_symbols() == sorted(_cabi.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    assert _cabi.is_built(), "build the library first: make -C dynaflow_amd/csrc"
+    lib = ctypes.CDLL(_cabi.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+
+
+def test_version_arch_and_status_text():
+    lib = _cabi.load()
+    assert lib.dfhip_version() >= 1000
+    assert lib.dfhip_arch() == b"gfx950"
+    assert lib.dfhip_status_string(0) == b"ok"
+    assert b"null" in lib.dfhip_status_string(-1)
+    with pytest.raises(_cabi.KernelError) as err:
+        _cabi.check("dfhip_gemm_bf16_nt", -2)
+    assert "unsupported shape" in str(err.value)
+
+
+def test_argument_checks_run_before_any_launch():
+    lib = _cabi.load()
+    # null pointers and bad shapes are rejected on the host; nothing reaches a device
+    assert lib.dfhip_gemm_bf16_nt(None, 64, None, 64, None, 64, 1, 8, 64, None) == -1
+    assert lib.dfhip_gemm_bf16_nt(16, 64, 16, 64, 16, 64, 1, 8, 63, None) == -2      # K % 64
+    assert lib.dfhip_gemm_bf16_nt(16, 32, 16, 64, 16, 64, 1, 8, 64, None) == -3      # lda < K
+    assert lib.dfhip_gemm_bf16_nt(8, 64, 16, 64, 16, 64, 1, 8, 64, None) == -4       # alignment
+    assert lib.dfhip_gemm_bf16_nt_variant(16, 64, 16, 64, 16, 64, 1, 8, 64, 99, None) == -7
+    assert lib.dfhip_silu_mul_bf16(16, 8, 16, 8, 16, 8, 1, 7, 0, None) == -2
+    assert lib.dfhip_rmsnorm_bf16(16, None, 16, 16, None, 1, 20000, 1e-5, None) == -2
+    assert lib.dfhip_gemm_fp8_nt(16, 128, 16, 128, 16, 8, None, None, 1, 8, 128, None) == -1
+
+
+def test_operators_refuse_host_tensors():
+    from dynaflow_amd import ops
+
+    x = torch.randn(4, 64).bfloat16()
+    w = torch.randn(8, 64).bfloat16()
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        ops.linear(x, w)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        ops.silu_mul(x, x)
+
+
+def test_missing_library_is_loud(monkeypatch):
+    monkeypatch.setattr(_cabi, "_lib", None)
+    monkeypatch.setattr(_cabi, "LIB_PATH", "/nonexistent/libdynaflow_hip.so")
+    with pytest.raises(_cabi.KernelLibraryMissing):
+        _cabi.load()

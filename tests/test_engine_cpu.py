@@ -1,0 +1,216 @@
+"""Host logic of a forward on the recording device seam: the engine + shipped
+schedulers must produce the launch order and event chain the oracle derives,
+and the results of eager PyTorch on the unsplit input."""
+import asyncio
+
+import pytest
+import torch
+
+from dynaflow_amd.backend import make_backend
+from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
+from dynaflow_amd.interface import ExecutionContext, OpSchedulerBase, SplitConfig
+from dynaflow_amd.manager import DynaFlowManager
+from dynaflow_amd.mlp import SwiGLUMLP
+from dynaflow_amd.schedulers import MLPOverlapScheduler
+from dynaflow_amd.schedulers.mlp_overlap import mlp_split_rules, mlp_tag_rules
+from oracle import schedule_trace as ref
+
+
+def make_config(splits=2, **extra):
+    knobs = {"min_nano_split_tokens": 8, "dump_graph": False}
+    knobs.update(extra)
+    return DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", splits,
+                          InductorConfig(enabled=False), CUDAGraphConfig(enabled=False, capture_sizes=[64, 128]), knobs)
+
+
+def compile_mlp(cfg, tokens=64, hidden=32, inter=96, scheduler=None):
+    torch._dynamo.reset()
+    torch.manual_seed(0)
+    model = SwiGLUMLP(hidden, inter, dtype=torch.float32)
+    manager = DynaFlowManager()
+    x = torch.randn(tokens, hidden)
+    torch._dynamo.mark_dynamic(x, 0)
+    compiled = torch.compile(model, backend=make_backend(manager, cfg, scheduler), fullgraph=True)
+    manager.prepare(tokens, [tokens])  # not initialised yet: trivial split, used by the tracing call
+    with torch.no_grad():
+        compiled(x)
+    return model, manager, compiled, x
+
+
+def top_level(manager):
+    top = []
+    for node in manager.graph_module.graph.nodes:
+        if node.op == "placeholder":
+            top.append("in")
+        elif node.op == "call_module":
+            top.append(("mod", node.target))
+        elif node.op == "output":
+            top.append("out")
+        else:
+            top.append("fn")
+    return top
+
+
+@pytest.mark.parametrize("order,splits", [("staggered", 2), ("round_robin", 2), ("staggered", 4), ("round_robin", 3)])
+def test_launch_order_and_streams_match_oracle(host_device, order, splits):
+    cfg = make_config(splits, schedule=order, num_nano_batches=splits)
+    model, manager, compiled, x = compile_mlp(cfg, tokens=96)
+    split = manager.prepare(96, [96])
+    assert split.num_nano_batches == splits
+    host_device.log.clear()
+    with torch.no_grad():
+        y = compiled(x)
+    assert manager.cached_config is None, "the split is consumed by the forward"
+    torch.testing.assert_close(y, model(x), rtol=0, atol=0)
+
+    want = ref.simulate(top_level(manager), splits, order,
+                        lambda m: "side" if "tail" in getattr(manager.graph_module, m).tag else "main",
+                        caller_stream="default")
+    ranges = [(e[1], e[2]) for e in host_device.log if e[0] == "range"]
+    got_launches = [(name.rsplit("_", 1)[0][3:], int(name.rsplit("_", 1)[1]), stream) for name, stream in ranges]
+    assert got_launches == ref.launches(want)
+    assert manager.engine.issue_trace == [(m, b) for m, b, _ in ref.launches(want)]
+
+    # the full event chain: map event uids to nano-batches through the order of creation
+    kinds = [(e[0], e[2]) for e in host_device.log if e[0] in ("record", "wait")]
+    want_kinds = [("record" if e[0] == "record" else "wait", e[2]) for e in want if e[0] in ("record", "wait", "join")]
+    assert kinds == want_kinds
+    # a wait always refers to the event its nano-batch recorded last
+    last_record = {}
+    launch_iter = iter(ref.launches(want))
+    for e in host_device.log:
+        if e[0] == "record":
+            last_record[e[1]] = e[2]
+        elif e[0] == "wait":
+            assert e[1] in last_record, "waited on an event that was never recorded"
+
+
+def test_environment_is_drained(host_device):
+    cfg = make_config(2)
+    model, manager, compiled, x = compile_mlp(cfg)
+    manager.prepare(64, [64])
+    with torch.no_grad():
+        compiled(x)
+    assert manager.engine.last_env.live_entries() == []
+
+
+def test_single_batch_takes_fast_path_and_bypasses_scheduler(host_device):
+    cfg = make_config(2, min_nano_split_tokens=1000)
+    model, manager, compiled, x = compile_mlp(cfg)
+    split = manager.prepare(64, [64])
+    assert split.num_nano_batches == 1
+    host_device.log.clear()
+    with torch.no_grad():
+        y = compiled(x)
+    assert [e for e in host_device.log if e[0] == "range"] == []
+    torch.testing.assert_close(y, model(x), rtol=0, atol=0)
+
+
+def test_single_batch_through_scheduler_when_fallback_disallowed(host_device):
+    cfg = make_config(2, min_nano_split_tokens=1000)
+    model, manager, compiled, x = compile_mlp(cfg)
+    split = manager.prepare(64, [64])
+    split.allow_fallback = False
+    manager.override_split_config(split)
+    with torch.no_grad():
+        y = compiled(x)
+    assert manager.engine.issue_trace == [("submod_0", 0), ("submod_1", 0)]
+    torch.testing.assert_close(y, model(x), rtol=0, atol=0)
+
+
+def test_forward_without_prepare_fails(host_device):
+    cfg = make_config(2)
+    model, manager, compiled, x = compile_mlp(cfg)
+    with pytest.raises(AssertionError):
+        compiled(x)
+
+
+def test_uneven_split_rows_land_in_order(host_device):
+    cfg = make_config(2)
+    model, manager, compiled, x = compile_mlp(cfg, tokens=50)
+    manager.override_split_config(SplitConfig(2, [13, 37], [0, 13, 50], [13, 37], [13, 37], [0, 13, 50], False, False))
+    with torch.no_grad():
+        y = compiled(x)
+    torch.testing.assert_close(y, model(x), rtol=0, atol=0)
+
+
+def test_dryrun_returns_whole_batch(host_device):
+    cfg = make_config(2)
+    model, manager, compiled, x = compile_mlp(cfg)
+    split = manager.prepare(64, [64], is_dryrun=True)
+    assert split.is_dryrun and split.num_nano_batches == 1
+    with torch.no_grad():
+        y = compiled(x)
+    torch.testing.assert_close(y, model(x), rtol=0, atol=0)
+
+
+class _OutOfOrder(MLPOverlapScheduler):
+    async def schedule(self, context: ExecutionContext) -> None:
+        first = await context.pop(0)
+        await context.execute((first,))
+        second = await context.pop(0)
+        # executing the first handle again violates the per-nano-batch FIFO
+        await context.execute((first,))
+
+
+def test_out_of_order_execution_is_caught(host_device):
+    cfg = make_config(2)
+    model, manager, compiled, x = compile_mlp(cfg, scheduler=_OutOfOrder(cfg))
+    manager.prepare(64, [64])
+    with pytest.raises((AssertionError, KeyError)):
+        compiled(x)
+
+
+class _Substituting(MLPOverlapScheduler):
+    calls = 0
+
+    async def schedule(self, context: ExecutionContext) -> None:
+        live = list(range(context.split_config.num_nano_batches))
+        while live:
+            for b in list(live):
+                op = await context.pop(b)
+                if op is None:
+                    live.remove(b)
+                    continue
+                if "tail" in op.tag:
+                    def tail(gate, size, up, w_down):
+                        _Substituting.calls += 1
+                        assert isinstance(size, int) and gate.shape[0] == size
+                        return torch.nn.functional.linear(torch.nn.functional.silu(gate) * up, w_down)
+                    await context.execute((op,), tail)
+                else:
+                    await context.execute(op)  # a bare handle is accepted too
+
+
+def test_operator_substitution_gets_node_inputs_in_graph_order(host_device):
+    cfg = make_config(2)
+    model, manager, compiled, x = compile_mlp(cfg, scheduler=_Substituting(cfg))
+    manager.prepare(64, [64])
+    _Substituting.calls = 0
+    with torch.no_grad():
+        y = compiled(x)
+    assert _Substituting.calls == 2
+    torch.testing.assert_close(y, model(x), rtol=1e-6, atol=1e-6)
+
+
+class _Quitter(MLPOverlapScheduler):
+    async def schedule(self, context: ExecutionContext) -> None:
+        op = await context.pop(0)
+        await context.execute((op,))
+
+
+def test_scheduler_that_returns_early_leaves_engine_waiting(host_device):
+    """Failure detection on the host: the engine blocks on the execute queue; a
+    caller that bounds the forward with a time-out sees it."""
+    cfg = make_config(2)
+    model, manager, compiled, x = compile_mlp(cfg, scheduler=_Quitter(cfg))
+    split = manager.prepare(64, [64])
+
+    async def bounded():
+        args = (model.gate_proj.weight, 64, x, model.up_proj.weight, model.down_proj.weight)
+        placeholders = [n.name for n in manager.engine.placeholder_nodes]
+        assert len(placeholders) == len(args)
+        await asyncio.wait_for(manager._forward_async(args, {}, split), timeout=0.5)
+
+    with pytest.raises(asyncio.TimeoutError):
+        asyncio.run(bounded())

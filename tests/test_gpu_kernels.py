@@ -1,0 +1,224 @@
+"""Parity of every C-ABI kernel against the CPU oracle, on an MI355X.
+
+Integer / byte results (e4m3 codes, bf16 bit patterns of elementwise ops) are
+compared bit for bit, except where a transcendental is involved: SiLU uses expf,
+whose last-ulp rounding may differ between libm and the device library, so bf16
+outputs may differ by one ulp on a small fraction of elements.  GEMM results are
+compared as max|got - want| / max|want| with the tolerance of the precision:
+fp32 1e-5, bf16 2e-2, fp8 5e-2 (against the dequantised fp32 product).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import cref, mlp
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"fp32": 1e-5, "bf16": 2e-2, "fp8": 5e-2}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    from dynaflow_amd import _cabi, ops as _ops
+
+    _cabi.load()
+    return _ops
+
+
+def rel_err(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+
+
+def u16(t):
+    return t.contiguous().cpu().view(torch.int16).numpy().view(np.uint16)
+
+
+def from_u16(a):
+    return torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
+
+
+def ulp_diff(a, b):
+    return (a.cpu().view(torch.int16).int() - b.cpu().view(torch.int16).int()).abs()
+
+
+def randn(shape, seed, std=1.0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return torch.randn(shape, generator=g) * std
+
+
+def test_device_info(ops):
+    from dynaflow_amd import _cabi
+
+    info = _cabi.device_info(0)
+    assert info["arch_name"].startswith("gfx950")
+    assert info["compute_units"] == 256 and info["wavefront_size"] == 64
+    assert info["lds_bytes_per_block"] >= 160 * 1024
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 8, 64), (7, 24, 64), (128, 128, 128), (300, 264, 192), (257, 512, 256),
+                                   (512, 1032, 320)])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3])
+def test_gemm_bf16_against_c_oracle(ops, M, N, K, variant):
+    a = randn((M, K), 1).bfloat16()
+    w = randn((N, K), 2, 0.05).bfloat16()
+    want = from_u16(cref.gemm_nt_bf16(u16(a), u16(w)))
+    if variant < 0:
+        got = ops.linear(a.cuda(), w.cuda())
+    else:
+        got = ops.linear_variant(a.cuda(), w.cuda(), variant)
+    torch.cuda.synchronize()
+    assert got.shape == (M, N) and got.dtype == torch.bfloat16
+    assert rel_err(got.float(), want.float()) < TOL["bf16"]
+    # much tighter in practice: fp32 accumulation and one rounding, so each entry is within
+    # one bf16 ulp of the exact value, plus fp32 accumulation noise on entries that cancel
+    g, w_ = got.float().cpu(), want.float()
+    assert bool(((g - w_).abs() <= 2 ** -7 * w_.abs() + 2e-4 * w_.abs().max()).all())
+
+
+def test_gemm_bf16_row_strided_views_and_batched_input(ops):
+    a_full = randn((64, 512), 3).bfloat16().cuda()
+    w = randn((96, 256), 4, 0.05).bfloat16().cuda()
+    a = a_full[:, 128:384]  # row stride 512, 16-byte aligned start
+    got = ops.linear(a, w)
+    want = torch.nn.functional.linear(a.float().cpu(), w.float().cpu())
+    assert rel_err(got.float(), want) < TOL["bf16"]
+    a3 = randn((4, 16, 256), 5).bfloat16().cuda()
+    got3 = ops.linear(a3, w)
+    assert got3.shape == (4, 16, 96)
+    assert rel_err(got3.float(), torch.nn.functional.linear(a3.float().cpu(), w.float().cpu())) < TOL["bf16"]
+
+
+def test_gemm_bf16_is_linear_in_its_input(ops):
+    """Size-independent property at a large shape: (a1 + a2) W == a1 W + a2 W when the sums are exact."""
+    M, N, K = 2048, 4096, 4096
+    a1 = (torch.randint(-4, 5, (M, K), generator=torch.Generator().manual_seed(1)).float() / 4).bfloat16().cuda()
+    a2 = (torch.randint(-4, 5, (M, K), generator=torch.Generator().manual_seed(2)).float() / 4).bfloat16().cuda()
+    w = (torch.randint(-8, 9, (N, K), generator=torch.Generator().manual_seed(3)).float() / 64).bfloat16().cuda()
+    # small integers over powers of two: every product and partial sum is exact in fp32
+    y1, y2, y12 = ops.linear(a1, w).float(), ops.linear(a2, w).float(), ops.linear(a1 + a2, w).float()
+    torch.cuda.synchronize()
+    assert rel_err(y12, y1 + y2) < 2 ** -7
+    # and the exact value on a sample of entries
+    rows = torch.tensor([0, 1, 777, 2047])
+    want = (a1[rows].double().cpu() @ w.double().cpu().t())
+    assert rel_err(ops.linear(a1[rows].contiguous(), w).float(), want.bfloat16().float()) < 2 ** -7
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 4, 4), (5, 7, 12), (130, 129, 64), (256, 2816, 1024)])
+def test_gemm_f32(ops, M, N, K):
+    a = randn((M, K), 6)
+    w = randn((N, K), 7, 0.02)
+    want = torch.from_numpy(cref.gemm_nt_f32(a.numpy(), w.numpy())) if M * N * K < 5e7 else a.double() @ w.double().t()
+    got = ops.linear(a.cuda(), w.cuda())
+    assert got.dtype == torch.float32
+    assert rel_err(got, want) < TOL["fp32"]
+
+
+@pytest.mark.parametrize("M,D", [(1, 8), (3, 40), (128, 2816), (257, 14336)])
+@pytest.mark.parametrize("round_silu", [False, True])
+def test_silu_mul_bf16_bits(ops, M, D, round_silu):
+    g = randn((M, D), 8, 3.0).bfloat16()
+    u = randn((M, D), 9).bfloat16()
+    want = from_u16(cref.silu_mul_bf16(u16(g), u16(u), round_silu))
+    got = ops.silu_mul(g.cuda(), u.cuda(), round_silu)
+    d = ulp_diff(got, want)
+    assert d.max() <= 1 and (d > 0).float().mean() < 5e-3
+
+
+def test_silu_mul_special_values_and_packed_layout(ops):
+    vals = torch.tensor([0.0, -0.0, 1.0, -1.0, 20.0, -20.0, 88.0, -88.0, 100.0, -100.0, 3.0e38, -3.0e38,
+                         float("inf"), -float("inf"), 1e-30, -1e-30]).bfloat16()
+    g = vals.repeat(4, 1)
+    u = torch.full_like(g, 2.0)
+    want = from_u16(cref.silu_mul_bf16(u16(g), u16(u), False))
+    got = ops.silu_mul(g.cuda(), u.cuda(), False).cpu()
+    same = (got.view(torch.int16) == want.view(torch.int16)) | (torch.isnan(got.float()) & torch.isnan(want.float()))
+    assert bool(same.all()), (got, want)
+    # packed gate_up[M, 2D]: halves passed as row-strided views
+    packed = randn((33, 2 * 64), 10, 2.0).bfloat16().cuda()
+    got = ops.silu_mul(packed[:, :64], packed[:, 64:], False)
+    want = ops.silu_mul(packed[:, :64].contiguous(), packed[:, 64:].contiguous(), False)
+    assert torch.equal(got, want)
+
+
+def test_silu_mul_f32(ops):
+    g, u = randn((37, 100), 11, 3.0), randn((37, 100), 12)
+    got = ops.silu_mul(g.cuda(), u.cuda())
+    want = (g.double() / (1 + torch.exp(-g.double()))) * u.double()
+    assert rel_err(got, want) < TOL["fp32"]
+
+
+@pytest.mark.parametrize("M,H", [(1, 8), (5, 512), (64, 4096), (3, 16384)])
+def test_rms_norm(ops, M, H):
+    x = randn((M, H), 13).bfloat16()
+    w = (1 + 0.1 * randn((H,), 14)).bfloat16()
+    want = from_u16(cref.rmsnorm_bf16(u16(x), u16(w), 1e-5))
+    got = ops.rms_norm(x.cuda(), w.cuda(), 1e-5)
+    # the row sum of squares is reduced in a different order than the sequential C loop, so the
+    # scale can differ in its last bit; after the two roundings that is at most 2 bf16 ulps
+    d = ulp_diff(got, want)
+    assert d.max() <= 2 and (d > 0).float().mean() < 1e-2
+    res = randn((M, H), 15).bfloat16()
+    out, new_res = ops.add_rms_norm(x.cuda(), res.cuda(), w.cuda(), 1e-5)
+    want_out, want_res = mlp.rms_norm(x, w, 1e-5, residual=res)
+    assert torch.equal(new_res.cpu(), want_res)
+    assert ulp_diff(out, want_out).max() <= 2
+
+
+def test_transpose_weight(ops):
+    w = randn((200, 136), 16).bfloat16().cuda()
+    assert torch.equal(ops.transpose_weight(w), w.t().contiguous())
+
+
+@pytest.mark.parametrize("M,D", [(1, 8), (9, 72), (256, 1024)])
+def test_quant_fp8_codes_are_bit_exact(ops, M, D):
+    x = randn((M, D), 17, 2.5).bfloat16()
+    want_q, want_s = mlp.quant_e4m3(x)
+    q, s = ops.quant_fp8(x.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(s.cpu(), want_s)
+    got = q.cpu().view(torch.uint8)
+    same = (got == want_q) | ((got & 0x7F == 0) & (want_q & 0x7F == 0))
+    assert bool(same.all())
+    # all-zero input: scale floor, codes zero
+    q0, s0 = ops.quant_fp8(torch.zeros(2, 16, dtype=torch.bfloat16, device="cuda"))
+    assert s0.item() == pytest.approx(1e-12 / 448) and int(q0.view(torch.uint8).max()) & 0x7F == 0
+
+
+def test_silu_mul_quant_fp8(ops):
+    g = randn((130, 256), 18, 3.0).bfloat16()
+    u = randn((130, 256), 19).bfloat16()
+    act = ops.silu_mul(g.cuda(), u.cuda(), False)
+    want_q, want_s = mlp.quant_e4m3(act.cpu())
+    q, s = ops.silu_mul_quant_fp8(g.cuda(), u.cuda())
+    assert torch.equal(s.cpu(), want_s)
+    got = q.cpu().view(torch.uint8)
+    assert bool(((got == want_q) | ((got & 0x7F == 0) & (want_q & 0x7F == 0))).all())
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 8, 128), (65, 72, 256), (300, 264, 384), (512, 1024, 1024)])
+def test_gemm_fp8_against_dequantised_fp32(ops, M, N, K):
+    x = randn((M, K), 20).bfloat16()
+    w = randn((N, K), 21, 0.02).bfloat16()
+    xq, xs = mlp.quant_e4m3(x)
+    wq, ws = mlp.quant_e4m3_per_channel(w)
+    want = mlp.dequant(xq, xs) @ mlp.dequant(wq, ws).t()
+    got = ops.linear_fp8(xq.cuda().view(torch.float8_e4m3fn), wq.cuda().view(torch.float8_e4m3fn), xs.cuda(), ws.cuda())
+    assert got.dtype == torch.bfloat16 and got.shape == (M, N)
+    assert rel_err(got.float(), want) < 2 ** -7  # products of e4m3 values are exact in fp32; one bf16 rounding
+    # and the whole quantise->multiply chain against the unquantised product, at the fp8 tolerance
+    assert rel_err(got.float(), x.float() @ w.float().t()) < TOL["fp8"] * (1 if K >= 256 else 4)
+
+
+def test_kernel_errors_become_exceptions(ops):
+    from dynaflow_amd import _cabi
+
+    a = torch.zeros(4, 72, dtype=torch.bfloat16, device="cuda")  # K % 64 != 0
+    w = torch.zeros(8, 72, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(_cabi.KernelError):
+        ops.linear(a, w)
+    with pytest.raises(RuntimeError):
+        ops.linear(a, torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda"))

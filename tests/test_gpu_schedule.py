@@ -1,0 +1,195 @@
+"""The whole path on an MI355X: torch.compile backend -> manager -> engine ->
+scheduler -> HIP operators on two streams, against the CPU oracle."""
+import pytest
+import torch
+
+from oracle import mlp
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"fp32": 1e-5, "bf16": 2e-2, "fp8": 5e-2}
+
+
+def rel_err(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+
+
+def build(tokens, hidden, inter, dtype, splits=2, prenorm=False, **knobs):
+    from dynaflow_amd.backend import make_backend
+    from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
+    from dynaflow_amd.manager import DynaFlowManager
+    from dynaflow_amd.mlp import SwiGLUMLP
+
+    extra = {"min_nano_split_tokens": 1, "num_nano_batches": splits, "dump_graph": False}
+    extra.update(knobs)
+    cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", splits, InductorConfig(enabled=True),
+                         CUDAGraphConfig(enabled=False, capture_sizes=[tokens]), extra)
+    x, wg, wu, wd = mlp.make_inputs(tokens, hidden, inter, dtype, prenorm=prenorm)
+    model = SwiGLUMLP(hidden, inter, dtype=dtype, device="cuda")
+    with torch.no_grad():
+        model.gate_proj.weight.copy_(wg)
+        model.up_proj.weight.copy_(wu)
+        model.down_proj.weight.copy_(wd)
+    manager = DynaFlowManager()
+    torch._dynamo.reset()
+    xg = x.cuda()
+    torch._dynamo.mark_dynamic(xg, 0)
+    compiled = torch.compile(model, backend=make_backend(manager, cfg), fullgraph=True)
+    manager.prepare(tokens, [tokens])
+    with torch.no_grad():
+        compiled(xg)  # traces; runs the trivial split through the fast path
+    return manager, compiled, xg, (x, wg, wu, wd)
+
+
+def run(manager, compiled, xg, tokens, use_cudagraph=False):
+    split = manager.prepare(tokens, [tokens], use_cudagraph=use_cudagraph)
+    with torch.no_grad():
+        y = compiled(xg)
+    torch.cuda.synchronize()
+    return y, split
+
+
+def test_subgraphs_run_on_hip_operators():
+    from dynaflow_amd import ops
+
+    manager, compiled, xg, _ = build(256, 1024, 2816, torch.float32)
+    for name in ("submod_0", "submod_1"):
+        backend = manager.graph_module.__dict__[name]
+        targets = [n.target for n in backend.callable_dynamic.graph.nodes if n.op == "call_function"]
+        assert all(t in (ops.linear, ops.silu_mul) for t in targets), targets
+
+
+def test_config1_fp32_matches_cpu_reference_path():
+    """x[256,1024] fp32, I=2816, 2 x 128 tokens: the reference's CPU-runnable case."""
+    manager, compiled, xg, (x, wg, wu, wd) = build(256, 1024, 2816, torch.float32)
+    y, split = run(manager, compiled, xg, 256)
+    assert split.split_indices == [0, 128, 256]
+    want = mlp.mlp_schedule(x, wg, wu, wd, split.split_indices)
+    assert rel_err(y, want) < TOL["fp32"]
+    assert manager.engine.issue_trace == [("submod_0", 0), ("submod_1", 0), ("submod_0", 1), ("submod_1", 1)]
+
+
+@pytest.mark.parametrize("tokens,splits", [(512, 2), (500, 2), (384, 3), (96, 4)])
+def test_bf16_schedule_small(tokens, splits):
+    manager, compiled, xg, (x, wg, wu, wd) = build(tokens, 512, 1408, torch.bfloat16, splits=splits)
+    y, split = run(manager, compiled, xg, tokens)
+    assert split.num_nano_batches == splits
+    want = mlp.mlp_schedule(x, wg, wu, wd, split.split_indices)     # eager bf16 PyTorch on the CPU
+    assert rel_err(y.float(), want.float()) < TOL["bf16"]
+    exact = mlp.mlp_fp32_from(x, wg, wu, wd)                       # fp32 on the same bf16 operands
+    assert rel_err(y.float(), exact) < TOL["bf16"]
+
+
+def test_config2_full_size_properties():
+    """x[4096,4096] bf16 pre-normed, I=14336, 2 x 2048.  The CPU oracle takes too long at this
+    size for the whole output, so: (1) sampled rows against the oracle, (2) split == unsplit
+    through the HIP path, (3) serialised == overlapped bit for bit."""
+    manager, compiled, xg, (x, wg, wu, wd) = build(4096, 4096, 14336, torch.bfloat16, prenorm=True)
+    y, split = run(manager, compiled, xg, 4096)
+    assert split.split_indices == [0, 2048, 4096]
+    rows = torch.tensor([0, 1, 2047, 2048, 3000, 4095])
+    want = mlp.mlp_fp32_from(x[rows], wg, wu, wd)
+    assert rel_err(y[rows].float(), want) < TOL["bf16"]
+    # unsplit through the same kernels (single nano-batch fast path)
+    from dynaflow_amd.manager import trivial_split
+
+    manager.override_split_config(trivial_split(4096, [4096], False, False))
+    with torch.no_grad():
+        whole = compiled(xg)
+    torch.cuda.synchronize()
+    assert rel_err(y.float(), whole.float()) < 2 ** -6
+    # a second overlapped run is bit-identical (no race between the streams)
+    y2, _ = run(manager, compiled, xg, 4096)
+    assert torch.equal(y, y2)
+
+
+def test_serialized_schedule_is_bit_identical_to_overlapped():
+    m1, c1, xg1, _ = build(1024, 1024, 2816, torch.bfloat16)
+    y1, _ = run(m1, c1, xg1, 1024)
+    m2, c2, xg2, _ = build(1024, 1024, 2816, torch.bfloat16, serialize=True)
+    y2, _ = run(m2, c2, xg2, 1024)
+    assert torch.equal(y1, y2)
+
+
+def test_whole_schedule_graph_replay():
+    """One hipGraph for the whole two-stream schedule: every replay must equal the eager result,
+    with eager work and synchronisations between the replays."""
+    manager, compiled, xg, (x, wg, wu, wd) = build(1024, 1024, 2816, torch.bfloat16, whole_graph=True)
+    eager, _ = run(manager, compiled, xg, 1024, use_cudagraph=False)
+    eager = eager.clone()
+    for i in range(4):
+        y, _ = run(manager, compiled, xg, 1024, use_cudagraph=True)
+        assert torch.equal(y, eager), f"replay {i}"
+        junk = torch.randn(512, 512, device="cuda") @ torch.randn(512, 512, device="cuda")
+        torch.cuda.synchronize()
+    assert len(manager._schedule_graphs) == 1
+    # new input values in the captured tensor are picked up by the replay
+    new_x = torch.randn_like(xg)
+    xg.copy_(new_x)
+    y, _ = run(manager, compiled, xg, 1024, use_cudagraph=True)
+    want, _ = run(manager, compiled, xg, 1024, use_cudagraph=False)
+    assert torch.equal(y, want)
+    # an input living elsewhere is copied into the captured tensor first
+    other = torch.randn_like(xg)
+    y, _ = run(manager, compiled, other, 1024, use_cudagraph=True)
+    want, _ = run(manager, compiled, other, 1024, use_cudagraph=False)
+    assert torch.equal(y, want)
+
+
+def fp8_layer(tokens, hidden, inter):
+    from dynaflow_amd.fp8_mlp import Fp8SwiGLU
+
+    x, wg, wu, wd = mlp.make_inputs(tokens, hidden, inter, torch.bfloat16)
+    quantised = [mlp.quant_e4m3_per_channel(w) for w in (wg, wu, wd)]
+    buffers = []
+    for codes, scale in quantised:
+        buffers += [codes.cuda().view(torch.float8_e4m3fn), scale.cuda()]
+    return Fp8SwiGLU(*buffers), x, quantised, (wg, wu, wd)
+
+
+def test_fp8_layer_against_dequantised_reference():
+    """fp8 MLP (per-tensor activation scale, per-channel weight scale), 4 nano-batches issued directly."""
+    from dynaflow_amd.fp8_mlp import Fp8SwiGLU
+
+    layer, x, quantised, (wg, wu, wd) = fp8_layer(512, 1024, 2048)
+    split = [0, 128, 256, 384, 512]
+    y = layer.forward_schedule(x.cuda(), split)
+    torch.cuda.synchronize()
+    (wg_q, wg_s), (wu_q, wu_s), (wd_q, wd_s) = quantised
+    want = mlp.mlp_fp8_dequant_reference(x, wg_q, wg_s, wu_q, wu_s, wd_q, wd_s, split)
+    assert rel_err(y.float(), want.float()) < TOL["fp8"]
+    # the device-side weight quantiser agrees with the oracle's codec (up to last-bit division effects)
+    auto = Fp8SwiGLU.from_weights(wg.cuda(), wu.cuda(), wd.cuda())
+    agree = ((auto.w_gate_q.cpu().view(torch.uint8) & 0x7F) == (wg_q & 0x7F)).float().mean()
+    assert agree > 0.999 and torch.allclose(auto.w_gate_s.cpu(), wg_s, rtol=1e-6)
+
+
+def test_fp8_layer_through_the_manager_with_four_nano_batches():
+    from dynaflow_amd.backend import make_backend
+    from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
+    from dynaflow_amd.manager import DynaFlowManager
+
+    tokens = 512
+    layer, x, quantised, _ = fp8_layer(tokens, 1024, 2048)
+    cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", 4, InductorConfig(enabled=True),
+                         CUDAGraphConfig(enabled=False, capture_sizes=[tokens]),
+                         {"min_nano_split_tokens": 1, "num_nano_batches": 4, "dump_graph": False})
+    manager = DynaFlowManager()
+    torch._dynamo.reset()
+    xg = x.cuda()
+    torch._dynamo.mark_dynamic(xg, 0)
+    compiled = torch.compile(layer, backend=make_backend(manager, cfg), fullgraph=True)
+    with torch.no_grad():
+        manager.prepare(tokens, [tokens])
+        compiled(xg)
+        split = manager.prepare(tokens, [tokens])
+        y = compiled(xg)
+    torch.cuda.synchronize()
+    assert split.split_indices == [0, 128, 256, 384, 512]
+    assert manager.engine.issue_trace == [("submod_0", 0), ("submod_1", 0), ("submod_0", 1), ("submod_0", 2),
+                                          ("submod_0", 3), ("submod_1", 1), ("submod_1", 2), ("submod_1", 3)]
+    (wg_q, wg_s), (wu_q, wu_s), (wd_q, wd_s) = quantised
+    want = mlp.mlp_fp8_dequant_reference(x, wg_q, wg_s, wu_q, wu_s, wd_q, wd_s, split.split_indices)
+    assert rel_err(y.float(), want.float()) < TOL["fp8"]
+    assert torch.equal(y, layer.forward_schedule(xg, split.split_indices))

@@ -1,0 +1,64 @@
+"""The HIP lowering pass on traced graphs (graph surgery only; nothing runs)."""
+import torch
+
+from dynaflow_amd import matching, ops
+from dynaflow_amd.executor.hip_lowering import lower_to_hip
+from dynaflow_amd.mlp import SwiGLUMLP
+from dynaflow_amd.schedulers.mlp_overlap import mlp_split_rules
+
+
+def traced(dtype, hidden=64, inter=128):
+    captured = {}
+
+    def backend(gm, example_inputs):
+        captured["gm"] = gm
+        return gm
+
+    torch._dynamo.reset()
+    x = torch.randn(16, hidden).to(dtype)
+    torch._dynamo.mark_dynamic(x, 0)
+    torch.compile(SwiGLUMLP(hidden, inter, dtype=dtype), backend=backend, fullgraph=True)(x)
+    return matching.split_graph(captured["gm"], mlp_split_rules())
+
+
+def targets(gm):
+    return [n.target for n in gm.graph.nodes if n.op == "call_function"]
+
+
+def test_bf16_mlp_subgraphs_are_fully_lowered():
+    split = traced(torch.bfloat16)
+    head, stats0 = lower_to_hip(split.submod_0)
+    tail, stats1 = lower_to_hip(split.submod_1)
+    assert stats0 == {"linear": 2, "silu_mul": 0} and stats1 == {"linear": 1, "silu_mul": 1}
+    assert targets(head) == [ops.linear, ops.linear]
+    assert targets(tail) == [ops.silu_mul, ops.linear]
+    silu_mul = next(n for n in tail.graph.nodes if n.target is ops.silu_mul)
+    assert silu_mul.args[2] is True  # bf16: silu rounded before the product, like two aten kernels
+    # the original sub-graph is untouched
+    assert ops.linear not in targets(split.submod_0)
+
+
+def test_fp32_is_lowered_without_intermediate_rounding_flag():
+    split = traced(torch.float32)
+    tail, stats = lower_to_hip(split.submod_1)
+    assert stats == {"linear": 1, "silu_mul": 1}
+    silu_mul = next(n for n in tail.graph.nodes if n.target is ops.silu_mul)
+    assert silu_mul.args[2] is False
+
+
+def test_unsupported_shapes_stay_on_aten():
+    split = traced(torch.bfloat16, hidden=40, inter=72)  # K % 64 != 0
+    head, stats = lower_to_hip(split.submod_0)
+    assert stats["linear"] == 0
+    assert all(t is not ops.linear for t in targets(head))
+
+
+def test_lowered_graph_fails_loudly_on_the_host():
+    import pytest
+
+    split = traced(torch.bfloat16)
+    head, _ = lower_to_hip(split.submod_0)
+    x = torch.randn(16, 64).bfloat16()
+    w = torch.randn(128, 64).bfloat16()
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        head(x, 16, w, w)
