@@ -1,18 +1,39 @@
 // bf16 GEMM for gfx950:  C[M,N] = A[M,K] * W[N,K]^T, fp32 accumulate, bf16 out.
 //
-// Both operands are K-contiguous, which is the layout the 32x32x16 bf16 MFMA
-// wants: every lane feeds 8 consecutive k of one row.  A workgroup owns a
-// BM x BN tile of C and walks K in slabs of 64.  Each slab of A and W is
-// fetched with 16-byte global loads into registers while the previous slab is
-// being multiplied, then parked in LDS (two buffers, one barrier per slab).
-// LDS rows are padded from 128 to 144 bytes so that the 16-byte fragment reads
-// of 16 consecutive rows fall into 16 different 16-byte bank groups.
+// Both operands are K-contiguous, the layout the 32x32x16 bf16 MFMA wants: every
+// lane feeds 8 consecutive k of one row.  The MFMA is issued with W as its first
+// operand and A as its second, i.e. it produces the transposed 32x32 block; in the
+// accumulator layout of v_mfma_f32_32x32x16 a lane then holds ONE row m of C and
+// runs of 4 consecutive columns n.
 //
-// The MFMA is issued with W as its first operand and A as its second, i.e. it
-// produces the transposed 32x32 block.  In the accumulator layout of
-// v_mfma_f32_32x32x16 a lane then holds ONE row m of C and runs of 4
-// consecutive columns n, which lets the epilogue store 8 bytes per lane
-// instead of 2.
+// Two kernels:
+//
+// gemm_bf16_ring_kernel (the fast path, 256x256 tile, 4 waves of 128x128)
+//   * K is walked in slabs of 64.  A slab of A (256 rows x 128 bytes) and a slab of
+//     W are "halves" of 32 KiB each; halves are copied global->LDS by the DMA path
+//     (global_load_lds_dwordx4, no registers involved) into a ring of five 32 KiB
+//     units (160 KiB, the whole LDS), so that one and a half slabs are in flight
+//     while one slab is being multiplied.
+//   * LDS rows are 128 bytes with the 16-byte chunk index XOR-ed by (row/2)%8; the
+//     DMA writes 1 KiB (8 rows) per instruction contiguously, the swizzle is applied
+//     on the global side by choosing which chunk each lane fetches.  Fragment reads
+//     (ds_read_b128, row = lane%32, chunk = 2*ks + lane/32) are then conflict free.
+//   * one wave per SIMD means nothing hides a stall, so the loop body is pinned
+//     instruction by instruction: after every MFMA at most one LDS read or one DMA
+//     issue, fragments of k-step s+1 are read while step s multiplies, and the
+//     workgroup barrier that hands LDS units back sits between k-steps 2 and 3 with
+//     MFMAs already in the pipe.
+//   * the loop is branch free: halves past the end of K re-read the last slab into
+//     units nobody reads, so the count of outstanding DMA instructions is the same in
+//     every iteration (s_waitcnt vmcnt(8) before the barrier).
+//   * epilogue: each wave parks its 128x128 block in LDS and stores whole 256-byte
+//     row pieces (16 bytes per lane).
+//   * tiles are numbered so that the ~32 workgroups resident on one XCD form a
+//     4 (M) x 8 (N) block of tiles and share operand slabs in that XCD's L2.
+//
+// gemm_bf16_nt_kernel (generic, register staged, any tile shape of the template)
+//   16-byte global loads into registers while the previous slab multiplies, parked
+//   in two padded LDS buffers, one barrier per slab.  Used for small shapes.
 #include "dfhip_common.h"
 
 namespace {
@@ -173,6 +194,192 @@ gemm_bf16_nt_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
   }
 }
 
+
+// ------------------------------------------------------------------ ring kernel
+constexpr int RBM = 256, RBN = 256, RTHREADS = 256;
+constexpr int UNIT = 32768, NUNITS = 5, RING_LDS = UNIT * NUNITS;
+constexpr int GROUP_M = 4;   // tiles of one XCD are walked in panels of GROUP_M tile rows
+constexpr int EROW = 272;    // padded row of the epilogue staging area (bytes)
+
+// One LDS-DMA instruction: 64 lanes x 16 bytes from per-lane global addresses to
+// LDS[lds_addr + 16*lane].  The compiler does not see the memory effect; ordering
+// is kept by hand with s_waitcnt vmcnt / s_barrier below.
+DFHIP_DEVICE void dma16(uint32_t lds_addr, const void* g) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(g)
+               : "memory", "m0");
+}
+template <int N>
+DFHIP_DEVICE void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+DFHIP_DEVICE void workgroup_barrier() { asm volatile("s_barrier" ::: "memory"); }
+#define DFHIP_PIN __builtin_amdgcn_sched_barrier(0)
+
+__global__ void __launch_bounds__(RTHREADS)
+gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, uint16_t* __restrict__ C,
+                      int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave & 1, wave_n = wave >> 1;
+
+  // tile order: XCD-contiguous ranges, inside a range panels of GROUP_M tile rows, m fastest
+  const int tile = remap_xcd(blockIdx.x, tiles_m * tiles_n);
+  const int per_panel = GROUP_M * tiles_n;
+  const int first_m = (tile / per_panel) * GROUP_M;
+  const int rows_in_panel = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+  const int in_panel = tile % per_panel;
+  const int m0 = (first_m + in_panel % rows_in_panel) * RBM;
+  const int n0 = (in_panel / rows_in_panel) * RBN;
+  const int KT = K / BK;
+
+  // DMA sources: instruction t of this wave covers rows (wave*8+t)*8 .. +8 of a half;
+  // lane -> (row, chunk ^ swizzle(row)) so that LDS slot `lane` holds the swizzled chunk
+  const uint8_t* a_src[8];
+  const uint8_t* w_src[8];
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    const int row = (wave * 8 + t) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    int ar = m0 + row; ar = ar < M ? ar : M - 1;   // rows past the edge re-read the last row; never stored
+    int wr = n0 + row; wr = wr < N ? wr : N - 1;
+    a_src[t] = reinterpret_cast<const uint8_t*>(A + (int64_t)ar * lda + chunk * 8);
+    w_src[t] = reinterpret_cast<const uint8_t*>(W + (int64_t)wr * ldw + chunk * 8);
+  }
+  const uint32_t wave_lds = wave * 8 * 1024;
+  auto dma_a = [&](int t, int slab, int unit) {
+    const int s = slab < KT ? slab : KT - 1;
+    dma16(unit * UNIT + wave_lds + t * 1024, a_src[t] + (int64_t)s * (BK * 2));
+  };
+  auto dma_w = [&](int t, int slab, int unit) {
+    const int s = slab < KT ? slab : KT - 1;
+    dma16(unit * UNIT + wave_lds + t * 1024, w_src[t] + (int64_t)s * (BK * 2));
+  };
+
+  const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
+  int koff[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) koff[ks] = ((2 * ks + fhalf) ^ fswz) * 16;
+  const int a_lane = (wave_m * 128 + frow) * 128, w_lane = (wave_n * 128 + frow) * 128;
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  // halves in issue order: A(0) W(0) A(1) W(1) A(2) ...; half h lives in unit h % 5
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_a(t, 0, 0);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_w(t, 0, 1);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_a(t, 1, 2);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_w(t, 1, 3);
+  wait_vmcnt<16>();   // slab 0 has landed; slab 1 may still be in flight
+  workgroup_barrier();
+
+  bf16x8 fa[2][4], fw[2][4];
+  auto read_frag = [&](int idx, int ks, int slot, int unit_a, int unit_w) {  // idx 0..3: A block, 4..7: W block
+    if (idx < 4)
+      fa[slot][idx] = *reinterpret_cast<const bf16x8*>(smem + unit_a * UNIT + a_lane + koff[ks] + idx * 4096);
+    else
+      fw[slot][idx - 4] = *reinterpret_cast<const bf16x8*>(smem + unit_w * UNIT + w_lane + koff[ks] + (idx - 4) * 4096);
+  };
+  auto mfma = [&](int q, int slot) {
+    const int i = q >> 2, j = q & 3;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
+  };
+
+  int ua = 0, uw = 1;   // units of the slab being multiplied
+  int ia = 4, iw = 0;   // units that A(kt+2) and W(kt+2) go to
+#pragma unroll
+  for (int idx = 0; idx < 8; ++idx) read_frag(idx, 0, 0, ua, uw);
+  for (int kt = 0; kt < KT; ++kt) {
+    // k-step 0: fragments of step 1 behind MFMAs 0..7, DMA of A(kt+2) behind MFMAs 8..15
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      mfma(q, 0);
+      if (q < 8) read_frag(q, 1, 1, ua, uw); else dma_a(q - 8, kt + 2, ia);
+      DFHIP_PIN;
+    }
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      mfma(q, 1);
+      if (q < 8) read_frag(q, 2, 0, ua, uw);
+      DFHIP_PIN;
+    }
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      mfma(q, 0);
+      if (q < 8) read_frag(q, 3, 1, ua, uw);
+      DFHIP_PIN;
+    }
+    // every LDS read of slab kt has been issued; once they have landed its two units are free.
+    // Slab kt+1 must have landed too: A(kt+1) was issued an iteration ago, W(kt+1) in the last
+    // k-step 3; only the 8 instructions of A(kt+2) may still be in flight.
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    wait_vmcnt<8>();
+    workgroup_barrier();
+    int na = ua + 2; if (na >= NUNITS) na -= NUNITS;
+    int nw = uw + 2; if (nw >= NUNITS) nw -= NUNITS;
+    // k-step 3: DMA of W(kt+2) into the unit A(kt) just left, then fragments of slab kt+1, step 0
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      mfma(q, 1);
+      if (q < 8) dma_w(q, kt + 2, iw); else read_frag(q - 8, 0, 0, na, nw);
+      DFHIP_PIN;
+    }
+    ua = na; uw = nw;
+    ia += 2; if (ia >= NUNITS) ia -= NUNITS;
+    iw += 2; if (iw >= NUNITS) iw -= NUNITS;
+  }
+  wait_vmcnt<0>();      // the padding halves issued by the last iterations
+  workgroup_barrier();  // other waves may still be reading fragments where this wave parks its block
+
+  uint8_t* park = smem + wave * (128 * EROW);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 v;
+        v[0] = pack2_bf16(acc[i][j][4 * g + 0], acc[i][j][4 * g + 1]);
+        v[1] = pack2_bf16(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+        *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * EROW + (j * 32 + g * 8 + fhalf * 4) * 2) = v;
+      }
+  DFHIP_PIN;
+  const int m_base = m0 + wave_m * 128, n_base = n0 + wave_n * 128;
+#pragma unroll 4
+  for (int p = 0; p < 32; ++p) {
+    const int id = p * 64 + lane;
+    const int row = id >> 4, c = id & 15;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * EROW + c * 16);
+    const int m = m_base + row, n = n_base + c * 8;
+    if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;  // N % 8 == 0
+  }
+}
+
+int launch_ring(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K,
+                hipStream_t stream) {
+  static bool lds_opted_in = false;
+  if (!lds_opted_in) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_ring_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, RING_LDS) != hipSuccess)
+      return DFHIP_ERR_LAUNCH;
+    lds_opted_in = true;
+  }
+  const int tiles_m = (M + RBM - 1) / RBM, tiles_n = (N + RBN - 1) / RBN;
+  hipLaunchKernelGGL(gemm_bf16_ring_kernel, dim3(tiles_m * tiles_n), dim3(RTHREADS), RING_LDS, stream,
+                     static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W), static_cast<uint16_t*>(C), M, N,
+                     K, lda, ldw, ldc, tiles_m, tiles_n);
+  return dfhip_check_launch();
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 int launch(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
            int K, hipStream_t stream) {
@@ -211,7 +418,8 @@ extern "C" int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void
   if (int rc = check_args(A, lda, W, ldw, C, ldc, M, N, K)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (variant) {
-    case 0: return launch<256, 256, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
+    case 0: return launch_ring(A, lda, W, ldw, C, ldc, M, N, K, s);
+    case 4: return launch<256, 256, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 1: return launch<256, 256, 2, 4>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 2: return launch<128, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 3: return launch<256, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
@@ -221,10 +429,10 @@ extern "C" int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void
 
 extern "C" int dfhip_gemm_bf16_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                                   int64_t ldc, int M, int N, int K, dfhip_stream_t stream) {
-  // Big tiles when they still give the 256 CUs at least one tile each.
+  // The 256x256 ring kernel whenever the problem has at least half a tile of rows and enough
+  // tiles to occupy a good part of the 256 CUs; the small register-staged tile otherwise.
   const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
   int variant = 2;
-  if (M > 128 && big_tiles >= 256) variant = 0;
-  else if (M > 128 && (int64_t)((M + 255) / 256) * ((N + 127) / 128) >= 192) variant = 3;
+  if (M > 128 && N > 128 && big_tiles >= 64) variant = 0;
   return dfhip_gemm_bf16_nt_variant(A, lda, W, ldw, C, ldc, M, N, K, variant, stream);
 }

@@ -78,8 +78,9 @@ int dfhip_gemm_bf16_nt(const void* A, int64_t lda, const void* W, int64_t ldw, v
                        int64_t ldc, int M, int N, int K, dfhip_stream_t stream);
 
 /* Same contraction with an explicit kernel variant, for tuning and tests.
- * variant: 0 = 256x256 tile / 4 waves, 1 = 256x256 / 8 waves,
- *          2 = 128x128 / 4 waves, 3 = 256x128 / 4 waves. */
+ * variant: 0 = 256x256 tile, LDS-DMA ring (the fast path);
+ *          register-staged tiles: 1 = 256x256 / 8 waves, 2 = 128x128 / 4 waves,
+ *          3 = 256x128 / 4 waves, 4 = 256x256 / 4 waves. */
 int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                                int64_t ldc, int M, int N, int K, int variant,
                                dfhip_stream_t stream);

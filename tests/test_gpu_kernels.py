@@ -60,7 +60,7 @@ def test_device_info(ops):
 
 @pytest.mark.parametrize("M,N,K", [(1, 8, 64), (7, 24, 64), (128, 128, 128), (300, 264, 192), (257, 512, 256),
                                    (512, 1032, 320)])
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4])
 def test_gemm_bf16_against_c_oracle(ops, M, N, K, variant):
     a = randn((M, K), 1).bfloat16()
     w = randn((N, K), 2, 0.05).bfloat16()
