@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_int64, c_uint32, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_uint32, c_void_p
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libdynaflow_hip.so"
@@ -54,6 +54,12 @@ SIGNATURES: dict[str, tuple] = {
     "dfhip_gemm_bf16_nt_variant": (
         c_int,
         [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, c_int, _P],
+    ),
+    "dfhip_gemm_bf16_plan": (c_int, [c_int, c_int, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
+    "dfhip_gemm_bf16_splitk_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "dfhip_gemm_bf16_nt_splitk": (
+        c_int,
+        [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, c_int, _P, c_size_t, _P],
     ),
     "dfhip_gemm_f32_nt": (c_int, [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P]),
     "dfhip_gemm_fp8_nt": (

@@ -213,25 +213,47 @@ DFHIP_DEVICE void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 DFHIP_DEVICE void workgroup_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+// 16-byte store / load that is coherent across the XCDs (sc1: written through to, and read
+// from, the memory side instead of the XCD-private L2).  Used for split-K partial blocks so
+// that no L2-wide write-back or invalidate is needed to hand them from one XCD to another.
+DFHIP_DEVICE void store_f32x4_device_coherent(f32x4* p, f32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+DFHIP_DEVICE f32x4 load_f32x4_device_coherent(const f32x4* p) {
+  f32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+// The loads above are invisible to the compiler's own wait-count bookkeeping: a value may only
+// be used after this, which ties the wait to the register so that the use cannot move above it.
+DFHIP_DEVICE void wait_loaded(f32x4& v) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(v)::"memory"); }
 #define DFHIP_PIN __builtin_amdgcn_sched_barrier(0)
 
 __global__ void __launch_bounds__(RTHREADS)
 gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, uint16_t* __restrict__ C,
-                      int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n) {
+                      int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n,
+                      int split_k, float* __restrict__ partials, int* __restrict__ arrivals) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave & 1, wave_n = wave >> 1;
 
   // tile order: XCD-contiguous ranges, inside a range panels of GROUP_M tile rows, m fastest
-  const int tile = remap_xcd(blockIdx.x, tiles_m * tiles_n);
+  // with split-K the parts of one tile are neighbours in launch order
+  const int work = remap_xcd(blockIdx.x, tiles_m * tiles_n * split_k);
+  const int tile = work / split_k;
+  const int part = work - tile * split_k;
   const int per_panel = GROUP_M * tiles_n;
   const int first_m = (tile / per_panel) * GROUP_M;
   const int rows_in_panel = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
   const int in_panel = tile % per_panel;
   const int m0 = (first_m + in_panel % rows_in_panel) * RBM;
   const int n0 = (in_panel / rows_in_panel) * RBN;
-  const int KT = K / BK;
+  // this workgroup multiplies slabs [slab0, slab0 + KT) of the K / 64 slabs
+  const int slabs_total = K / BK;
+  const int slab0 = (int)((int64_t)slabs_total * part / split_k);
+  const int KT = (int)((int64_t)slabs_total * (part + 1) / split_k) - slab0;
 
   // DMA sources: instruction t of this wave covers rows (wave*8+t)*8 .. +8 of a half;
   // lane -> (row, chunk ^ swizzle(row)) so that LDS slot `lane` holds the swizzled chunk
@@ -248,11 +270,11 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   }
   const uint32_t wave_lds = wave * 8 * 1024;
   auto dma_a = [&](int t, int slab, int unit) {
-    const int s = slab < KT ? slab : KT - 1;
+    const int s = slab0 + (slab < KT ? slab : KT - 1);
     dma16(unit * UNIT + wave_lds + t * 1024, a_src[t] + (int64_t)s * (BK * 2));
   };
   auto dma_w = [&](int t, int slab, int unit) {
-    const int s = slab < KT ? slab : KT - 1;
+    const int s = slab0 + (slab < KT ? slab : KT - 1);
     dma16(unit * UNIT + wave_lds + t * 1024, w_src[t] + (int64_t)s * (BK * 2));
   };
 
@@ -340,6 +362,66 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   wait_vmcnt<0>();      // the padding halves issued by the last iterations
   workgroup_barrier();  // other waves may still be reading fragments where this wave parks its block
 
+  if (split_k > 1) {
+    // Every part leaves its fp32 block in `partials` and takes a ticket; the part that draws the
+    // last ticket adds all parts up in part order (so the sum does not depend on who came last)
+    // and writes the tile.  Nobody waits for anybody.
+    f32x4* mine = reinterpret_cast<f32x4*>(partials) + ((int64_t)tile * split_k + part) * (64 * RTHREADS) + tid;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+          store_f32x4_device_coherent(mine + ((i * 4 + j) * 4 + g) * RTHREADS, v);
+        }
+    wait_vmcnt<0>();       // the write-through stores have completed before the ticket is drawn
+    __syncthreads();
+    int* ticket_cell = reinterpret_cast<int*>(smem);
+    if (tid == 0) *ticket_cell = atomicAdd(arrivals + tile, 1);
+    __syncthreads();
+    const int ticket = *ticket_cell;
+    __syncthreads();
+    if (ticket != split_k - 1) return;
+    if (tid == 0) atomicExch(arrivals + tile, 0);   // ready for the next launch
+    // sum the parts in part order, 16 chunks (one row of MFMA blocks) at a time; the own part
+    // comes from the registers, the others through device-coherent loads issued back to back
+    const f32x4* all = reinterpret_cast<const f32x4*>(partials) + (int64_t)tile * split_k * (64 * RTHREADS) + tid;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f32x4 sum[16];
+#pragma unroll
+      for (int c = 0; c < 16; ++c) sum[c] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      for (int p = 0; p < split_k; ++p) {
+        if (p == part) {
+#pragma unroll
+          for (int c = 0; c < 16; ++c) {
+            const int j = c >> 2, g = c & 3;
+            sum[c] += f32x4{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+          }
+        } else {
+          f32x4 v[16];
+#pragma unroll
+          for (int c = 0; c < 16; ++c)
+            v[c] = load_f32x4_device_coherent(all + ((int64_t)p * 64 + i * 16 + c) * RTHREADS);
+#pragma unroll
+          for (int c = 0; c < 16; ++c) wait_loaded(v[c]);
+#pragma unroll
+          for (int c = 0; c < 16; ++c) sum[c] += v[c];
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < 16; ++c) {
+        const int j = c >> 2, g = c & 3;
+        acc[i][j][4 * g] = sum[c][0];
+        acc[i][j][4 * g + 1] = sum[c][1];
+        acc[i][j][4 * g + 2] = sum[c][2];
+        acc[i][j][4 * g + 3] = sum[c][3];
+      }
+    }
+  }
+
   uint8_t* park = smem + wave * (128 * EROW);
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -365,7 +447,7 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
 }
 
 int launch_ring(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K,
-                hipStream_t stream) {
+                int split_k, void* workspace, hipStream_t stream) {
   static bool lds_opted_in = false;
   if (!lds_opted_in) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_ring_kernel),
@@ -374,9 +456,16 @@ int launch_ring(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
     lds_opted_in = true;
   }
   const int tiles_m = (M + RBM - 1) / RBM, tiles_n = (N + RBN - 1) / RBN;
-  hipLaunchKernelGGL(gemm_bf16_ring_kernel, dim3(tiles_m * tiles_n), dim3(RTHREADS), RING_LDS, stream,
+  // workspace layout: [tiles] arrival counters (padded to 256 bytes), then [tiles][split_k] fp32 blocks
+  int* arrivals = static_cast<int*>(workspace);
+  float* partials = nullptr;
+  if (split_k > 1) {
+    const size_t counter_bytes = (((size_t)tiles_m * tiles_n * sizeof(int)) + 255) & ~(size_t)255;
+    partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + counter_bytes);
+  }
+  hipLaunchKernelGGL(gemm_bf16_ring_kernel, dim3(tiles_m * tiles_n * split_k), dim3(RTHREADS), RING_LDS, stream,
                      static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W), static_cast<uint16_t*>(C), M, N,
-                     K, lda, ldw, ldc, tiles_m, tiles_n);
+                     K, lda, ldw, ldc, tiles_m, tiles_n, split_k, partials, arrivals);
   return dfhip_check_launch();
 }
 
@@ -418,7 +507,7 @@ extern "C" int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void
   if (int rc = check_args(A, lda, W, ldw, C, ldc, M, N, K)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (variant) {
-    case 0: return launch_ring(A, lda, W, ldw, C, ldc, M, N, K, s);
+    case 0: return launch_ring(A, lda, W, ldw, C, ldc, M, N, K, 1, nullptr, s);
     case 4: return launch<256, 256, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 1: return launch<256, 256, 2, 4>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 2: return launch<128, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
@@ -427,12 +516,48 @@ extern "C" int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void
   }
 }
 
+extern "C" int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* split_k) {
+  if (!variant || !split_k) return DFHIP_ERR_NULL_POINTER;
+  if (M < 1 || N < 1 || K < 1) return DFHIP_ERR_BAD_SHAPE;
+  // The 256x256 ring kernel whenever the problem has more than half a tile of rows and columns
+  // and enough tiles to occupy a good part of the 256 CUs; the small register-staged tile
+  // otherwise.  With at most half as many tiles as CUs, K is split so that every CU gets a part.
+  const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+  *variant = 2;
+  *split_k = 1;
+  if (M > 128 && N > 128 && big_tiles >= 32) {
+    *variant = 0;
+    int s = (int)(256 / big_tiles);
+    if (s > 8) s = 8;
+    while (s > 1 && K / BK < 16 * s) --s;   // keep at least 16 slabs per part
+    if (s > 1) *split_k = s;
+  }
+  return DFHIP_OK;
+}
+
 extern "C" int dfhip_gemm_bf16_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                                   int64_t ldc, int M, int N, int K, dfhip_stream_t stream) {
-  // The 256x256 ring kernel whenever the problem has at least half a tile of rows and enough
-  // tiles to occupy a good part of the 256 CUs; the small register-staged tile otherwise.
-  const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-  int variant = 2;
-  if (M > 128 && N > 128 && big_tiles >= 64) variant = 0;
+  int variant = 2, split_k = 1;
+  if (int rc = dfhip_gemm_bf16_plan(M, N, K, &variant, &split_k)) return rc;
   return dfhip_gemm_bf16_nt_variant(A, lda, W, ldw, C, ldc, M, N, K, variant, stream);
+}
+
+extern "C" size_t dfhip_gemm_bf16_splitk_workspace_bytes(int M, int N, int split_k) {
+  if (M < 1 || N < 1 || split_k < 2) return 0;
+  const size_t tiles = (size_t)((M + RBM - 1) / RBM) * ((N + RBN - 1) / RBN);
+  const size_t counter_bytes = ((tiles * sizeof(int)) + 255) & ~(size_t)255;
+  return counter_bytes + tiles * split_k * (size_t)RBM * RBN * sizeof(float);
+}
+
+extern "C" int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                                         int64_t ldc, int M, int N, int K, int split_k, void* workspace,
+                                         size_t workspace_bytes, dfhip_stream_t stream) {
+  if (int rc = check_args(A, lda, W, ldw, C, ldc, M, N, K)) return rc;
+  if (split_k < 1 || split_k > 8 || K / BK < split_k) return DFHIP_ERR_BAD_ARGUMENT;
+  if (split_k > 1) {
+    if (!workspace) return DFHIP_ERR_NULL_POINTER;
+    if (!dfhip_aligned16(workspace)) return DFHIP_ERR_BAD_ALIGNMENT;
+    if (workspace_bytes < dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k)) return DFHIP_ERR_BAD_ARGUMENT;
+  }
+  return launch_ring(A, lda, W, ldw, C, ldc, M, N, K, split_k, workspace, static_cast<hipStream_t>(stream));
 }

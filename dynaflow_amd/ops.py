@@ -20,6 +20,8 @@ dynaflow/runtime/engine.py:381.
 """
 from __future__ import annotations
 
+import os
+
 import torch
 
 from dynaflow_amd import _cabi
@@ -67,7 +69,33 @@ def _require_device(*tensors: torch.Tensor) -> None:
 
 
 # ---------------------------------------------------------------- linear
-def _linear_impl(x: torch.Tensor, weight: torch.Tensor, variant: int = -1) -> torch.Tensor:
+#: split-K workspaces, one per (device, stream): launches on one stream run one after the
+#: other, launches on different streams may overlap and must not share arrival counters
+_splitk_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+#: split K for shapes with too few tiles (DYNAFLOW_SPLIT_K=0 switches it off)
+SPLIT_K_ENABLED = os.environ.get("DYNAFLOW_SPLIT_K", "1") != "0"
+
+
+def _splitk_workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
+    key = (device.index or 0, stream)
+    ws = _splitk_workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("split-K workspace must exist before graph capture: run the shape eagerly once")
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        _splitk_workspaces[key] = ws
+    return ws
+
+
+def _plan_bf16(lib, M: int, N: int, K: int) -> tuple[int, int]:
+    import ctypes
+
+    variant, split_k = ctypes.c_int(0), ctypes.c_int(1)
+    _cabi.check("dfhip_gemm_bf16_plan", lib.dfhip_gemm_bf16_plan(M, N, K, ctypes.byref(variant), ctypes.byref(split_k)))
+    return variant.value, split_k.value
+
+
+def _linear_impl(x: torch.Tensor, weight: torch.Tensor, variant: int = -1, split_k_allowed: bool = True) -> torch.Tensor:
     _require_device(x, weight)
     lib = _cabi.load()
     if weight.dim() != 2 or x.shape[-1] != weight.shape[1]:
@@ -79,16 +107,29 @@ def _linear_impl(x: torch.Tensor, weight: torch.Tensor, variant: int = -1) -> to
     out = torch.empty((M, N), dtype=x.dtype, device=x.device)
     if M > 0:
         if x.dtype == torch.bfloat16:
+            if variant == -2:
+                split_k_allowed, variant = False, -1
             if variant >= 0:
                 rc = lib.dfhip_gemm_bf16_nt_variant(
                     a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), N, M, N, K, variant, _stream()
                 )
                 _cabi.check("dfhip_gemm_bf16_nt_variant", rc)
             else:
-                rc = lib.dfhip_gemm_bf16_nt(
-                    a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), N, M, N, K, _stream()
-                )
-                _cabi.check("dfhip_gemm_bf16_nt", rc)
+                _, split_k = _plan_bf16(lib, M, N, K)
+                if split_k > 1 and split_k_allowed and SPLIT_K_ENABLED:
+                    stream = _stream()
+                    nbytes = lib.dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k)
+                    ws = _splitk_workspace(x.device, stream, nbytes)
+                    rc = lib.dfhip_gemm_bf16_nt_splitk(
+                        a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), N, M, N, K, split_k,
+                        ws.data_ptr(), ws.numel(), stream,
+                    )
+                    _cabi.check("dfhip_gemm_bf16_nt_splitk", rc)
+                else:
+                    rc = lib.dfhip_gemm_bf16_nt(
+                        a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), N, M, N, K, _stream()
+                    )
+                    _cabi.check("dfhip_gemm_bf16_nt", rc)
         elif x.dtype == torch.float32:
             rc = lib.dfhip_gemm_f32_nt(
                 a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), N, M, N, K, _stream()

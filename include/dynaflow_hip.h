@@ -85,6 +85,26 @@ int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void* W, int64_
                                int64_t ldc, int M, int N, int K, int variant,
                                dfhip_stream_t stream);
 
+/* The kernel choice dfhip_gemm_bf16_nt makes for a shape (variant as above) and
+ * the split_k a caller with a workspace should pass to dfhip_gemm_bf16_nt_splitk
+ * (1 = no split). */
+int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* split_k);
+
+/* Split-K flavour of the fast path for shapes with few output tiles (the down
+ * projection: [2048,14336] x [4096,14336]^T has 128 tiles of 256x256 for 256
+ * compute units).  Each tile is computed by `split_k` workgroups over disjoint
+ * K ranges; every part leaves its fp32 block in `workspace`, the part that
+ * arrives last adds the blocks up in part order (deterministic) and writes C.
+ * No workgroup waits for another.  `workspace` (device memory, 16-byte aligned,
+ * at least dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k) bytes) starts
+ * with the per-tile arrival counters, which must be ZERO before the first use
+ * and are left zero by every launch; launches that may overlap in time need
+ * workspaces of their own.  1 <= split_k <= 8, split_k <= K / 64. */
+size_t dfhip_gemm_bf16_splitk_workspace_bytes(int M, int N, int split_k);
+int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                              int64_t ldc, int M, int N, int K, int split_k, void* workspace,
+                              size_t workspace_bytes, dfhip_stream_t stream);
+
 /* fp32 in / fp32 accumulate / fp32 out (the CPU-sized fp32 configuration).
  * Requires K % 4 == 0, 16-byte aligned pointers, lda/ldw % 4 == 0. */
 int dfhip_gemm_f32_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,

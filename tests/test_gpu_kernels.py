@@ -222,3 +222,61 @@ def test_kernel_errors_become_exceptions(ops):
         ops.linear(a, w)
     with pytest.raises(RuntimeError):
         ops.linear(a, torch.zeros(8, 64, dtype=torch.bfloat16, device="cuda"))
+
+
+@pytest.mark.parametrize("M,N,K,split_k", [(300, 264, 512, 2), (300, 264, 512, 3), (256, 512, 512, 8), (513, 256, 1024, 4)])
+def test_gemm_bf16_split_k_against_c_oracle(ops, M, N, K, split_k):
+    """Split-K through the C ABI: parts leave fp32 blocks in a workspace, the last arriver sums them."""
+    from dynaflow_amd import _cabi
+
+    lib = _cabi.load()
+    a = randn((M, K), 31).bfloat16()
+    w = randn((N, K), 32, 0.05).bfloat16()
+    want = from_u16(cref.gemm_nt_bf16(u16(a), u16(w))).float()
+    ag, wg = a.cuda(), w.cuda()
+    nbytes = lib.dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k)
+    assert nbytes > 0
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    outs = []
+    for _ in range(3):  # the arrival counters must come back to zero after every launch
+        out = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+        rc = lib.dfhip_gemm_bf16_nt_splitk(ag.data_ptr(), K, wg.data_ptr(), K, out.data_ptr(), N, M, N, K, split_k,
+                                           ws.data_ptr(), nbytes, stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        outs.append(out)
+    g = outs[0].float().cpu()
+    assert bool(((g - want).abs() <= 2 ** -7 * want.abs() + 2e-4 * want.abs().max()).all())
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])
+    tiles = ((M + 255) // 256) * ((N + 255) // 256)
+    assert int(ws[: tiles * 4].view(torch.int32).abs().sum()) == 0
+    # too small a workspace and too many parts are refused
+    assert lib.dfhip_gemm_bf16_nt_splitk(ag.data_ptr(), K, wg.data_ptr(), K, out.data_ptr(), N, M, N, K, split_k,
+                                         ws.data_ptr(), 16, stream) == -7
+    assert lib.dfhip_gemm_bf16_nt_splitk(ag.data_ptr(), K, wg.data_ptr(), K, out.data_ptr(), N, M, N, K, 9,
+                                         ws.data_ptr(), nbytes, stream) == -7
+
+
+def test_down_projection_shape_uses_split_k_and_matches_unsplit(ops):
+    """[2048,14336] x [4096,14336]^T has 128 tiles for 256 CUs: the plan splits K in two."""
+    import ctypes
+    from dynaflow_amd import _cabi
+
+    lib = _cabi.load()
+    v, s = ctypes.c_int(), ctypes.c_int()
+    assert lib.dfhip_gemm_bf16_plan(2048, 4096, 14336, ctypes.byref(v), ctypes.byref(s)) == 0
+    assert (v.value, s.value) == (0, 2)
+    assert lib.dfhip_gemm_bf16_plan(2048, 14336, 4096, ctypes.byref(v), ctypes.byref(s)) == 0
+    assert (v.value, s.value) == (0, 1)
+    a = randn((2048, 14336), 33).bfloat16().cuda()
+    w = randn((4096, 14336), 34, 0.02).bfloat16().cuda()
+    split = ops.linear(a, w)
+    again = ops.linear(a, w)
+    whole = ops.linear_variant(a, w, -2)   # same kernel, K not split
+    torch.cuda.synchronize()
+    assert torch.equal(split, again)
+    assert rel_err(split.float(), whole.float()) < 2 ** -7
+    rows = torch.tensor([0, 255, 256, 1023, 2047])
+    want = a[rows].double().cpu() @ w.double().cpu().t()
+    assert rel_err(split[rows].float(), want) < 2 ** -7
