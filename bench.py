@@ -36,6 +36,7 @@ if ROOT not in sys.path:
 TOKENS, HIDDEN, INTER, SPLITS = 4096, 4096, 14336, 2
 BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E
+GATE_GEMM_TRAFFIC_BYTES = 493.6e6  # measured with hardware counters; the summary is under profiles/
 METRIC = "MLP-layer tokens/s + overlap speedup vs serial, 8B-shape bf16, 1 MI355X"
 
 
@@ -45,6 +46,9 @@ def parse_args():
     p.add_argument("--steps", type=int, default=50)
     p.add_argument("--warmup", type=int, default=15)
     p.add_argument("--skip-cpu", action="store_true", help="leave out the host baseline (profiling runs)")
+    p.add_argument("--kernels-only", action="store_true",
+                   help="run only the single-kernel timing loops plus a 256 MiB device copy (used to calibrate "
+                        "FETCH_SIZE / WRITE_SIZE under rocprofv3 --pmc); prints the kernel figures as JSON")
     return p.parse_args()
 
 
@@ -103,6 +107,26 @@ def time_kernel(torch, fn, iters, warmup=5):
     stop.record()
     stop.synchronize()
     return start.elapsed_time(stop) / iters
+
+
+def single_kernels(torch, ops, x, weights, iters, calibration_copy=False):
+    """Average launch durations (ms) of the kernels of one nano-batch, each timed alone."""
+    mb = TOKENS // SPLITS
+    xb = x[:mb]
+    gate = ops.linear(xb, weights[0])
+    up = ops.linear(xb, weights[1])
+    act = ops.silu_mul(gate, up, True)
+    out = {
+        "gate_ms": time_kernel(torch, lambda: ops.linear(xb, weights[0]), iters),
+        "down_ms": time_kernel(torch, lambda: ops.linear(act, weights[2]), iters),
+        "silu_ms": time_kernel(torch, lambda: ops.silu_mul(gate, up, True), iters),
+        "blas_ms": time_kernel(torch, lambda: torch.nn.functional.linear(xb, weights[0]), iters),
+    }
+    if calibration_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        out["copy_256MiB_ms"] = time_kernel(torch, lambda: dst.copy_(src), iters)
+    return out
 
 
 def cpu_baseline(torch):
@@ -165,6 +189,10 @@ def main() -> int:
     x = x_cpu.cuda()
     weights = (wg.cuda(), wu.cuda(), wd.cuda())
 
+    if args.kernels_only:
+        print(json.dumps(single_kernels(torch, ops, x, weights, max(20, args.steps), calibration_copy=True)))
+        return 0
+
     # ---- the three ways of issuing the schedule
     m_ser, c_ser = build_path(torch, x, weights, serialize=True)
     ms_serial, y_serial = time_steps(torch, m_ser, c_ser, x, args.steps, args.warmup, use_graph=False)
@@ -181,16 +209,9 @@ def main() -> int:
     rel_err = ((y_graph[rows].float().cpu() - want).abs().max() / want.abs().max()).item()
 
     # ---- single kernels, HIP events on the launching stream
+    k = single_kernels(torch, ops, x, weights, max(20, args.steps))
+    ms_gate, ms_down, ms_silu, ms_blas = k["gate_ms"], k["down_ms"], k["silu_ms"], k["blas_ms"]
     mb = TOKENS // SPLITS
-    xb = x[:mb]
-    gate = ops.linear(xb, weights[0])
-    up = ops.linear(xb, weights[1])
-    act = ops.silu_mul(gate, up, True)
-    iters = max(20, args.steps)
-    ms_gate = time_kernel(torch, lambda: ops.linear(xb, weights[0]), iters)
-    ms_down = time_kernel(torch, lambda: ops.linear(act, weights[2]), iters)
-    ms_silu = time_kernel(torch, lambda: ops.silu_mul(gate, up, True), iters)
-    ms_blas = time_kernel(torch, lambda: torch.nn.functional.linear(xb, weights[0]), iters)
     gemm_flops = 2.0 * mb * HIDDEN * INTER          # one projection of one nano-batch
     silu_bytes = 3.0 * mb * INTER * 2               # read gate + up, write out
     layer_flops = 6.0 * TOKENS * HIDDEN * INTER
@@ -244,7 +265,10 @@ def main() -> int:
             "peak": BF16_MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": gemm_flops / (ms_gate * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
-            "traffic": None,
+            # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy of
+            # known size (fetch 370.7 MB + write 122.9 MB); algorithmic: 134.2 MB read + 58.7 MB written
+            "traffic": GATE_GEMM_TRAFFIC_BYTES,
+            "traffic_unit": "bytes per launch",
         },
     }
     if not args.skip_cpu:
