@@ -385,39 +385,31 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
     __syncthreads();
     if (ticket != split_k - 1) return;
     if (tid == 0) atomicExch(arrivals + tile, 0);   // ready for the next launch
-    // sum the parts in part order, 16 chunks (one row of MFMA blocks) at a time; the own part
-    // comes from the registers, the others through device-coherent loads issued back to back
+    // add the parts up in part order, 8 chunks (half a row of MFMA blocks) at a time; the own
+    // part is read back like the others so that the accumulators can start from zero
     const f32x4* all = reinterpret_cast<const f32x4*>(partials) + (int64_t)tile * split_k * (64 * RTHREADS) + tid;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      f32x4 sum[16];
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int c = 0; c < 16; ++c) sum[c] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-      for (int p = 0; p < split_k; ++p) {
-        if (p == part) {
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-          for (int c = 0; c < 16; ++c) {
-            const int j = c >> 2, g = c & 3;
-            sum[c] += f32x4{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-          }
-        } else {
-          f32x4 v[16];
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    for (int p = 0; p < split_k; ++p) {
 #pragma unroll
-          for (int c = 0; c < 16; ++c)
-            v[c] = load_f32x4_device_coherent(all + ((int64_t)p * 64 + i * 16 + c) * RTHREADS);
+      for (int h = 0; h < 8; ++h) {   // chunks 8h .. 8h+7: blocks (i, j) = (h/2, 2*(h%2) + 0..1)
+        f32x4 v[8];
 #pragma unroll
-          for (int c = 0; c < 16; ++c) wait_loaded(v[c]);
+        for (int c = 0; c < 8; ++c) v[c] = load_f32x4_device_coherent(all + ((int64_t)p * 64 + h * 8 + c) * RTHREADS);
 #pragma unroll
-          for (int c = 0; c < 16; ++c) sum[c] += v[c];
+        for (int c = 0; c < 8; ++c) wait_loaded(v[c]);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          const int i = h >> 1, j = (h & 1) * 2 + (c >> 2), g = c & 3;
+          acc[i][j][4 * g] += v[c][0];
+          acc[i][j][4 * g + 1] += v[c][1];
+          acc[i][j][4 * g + 2] += v[c][2];
+          acc[i][j][4 * g + 3] += v[c][3];
         }
-      }
-#pragma unroll
-      for (int c = 0; c < 16; ++c) {
-        const int j = c >> 2, g = c & 3;
-        acc[i][j][4 * g] = sum[c][0];
-        acc[i][j][4 * g + 1] = sum[c][1];
-        acc[i][j][4 * g + 2] = sum[c][2];
-        acc[i][j][4 * g + 3] = sum[c][3];
       }
     }
   }
