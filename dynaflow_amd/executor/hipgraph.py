@@ -71,6 +71,9 @@ class CUDAGraphWrapper:
             with torch.cuda.graph(graph, pool=_global_pool.get_pool(handle.batch_idx)):
                 out = self.runnable(*args, **kwargs)
             self._entries[key] = {"graph": graph, "out": out, "inputs": _tensor_addresses(args)}
+            # capture records without running; replay once so that the dry-run's result is real
+            # (the reference hands back the unexecuted capture outputs, cudagraph.py:100-113)
+            graph.replay()
             return out
 
         if self.config.check_ptr_consistency and _tensor_addresses(args) != entry["inputs"]:

@@ -193,3 +193,63 @@ def test_fp8_layer_through_the_manager_with_four_nano_batches():
     want = mlp.mlp_fp8_dequant_reference(x, wg_q, wg_s, wu_q, wu_s, wd_q, wd_s, split.split_indices)
     assert rel_err(y.float(), want.float()) < TOL["fp8"]
     assert torch.equal(y, layer.forward_schedule(xg, split.split_indices))
+
+
+def test_piecewise_graphs_capture_in_dryrun_and_replay():
+    """Per-sub-graph hipGraphs as in the reference: captured for every (size, nano-batch index) during a
+    dry-run over fake nano-batches, replayed by the scheduled forward against per-nano-batch static buffers."""
+    from dynaflow_amd.backend import make_backend
+    from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
+    from dynaflow_amd.interface import SplitConfig
+    from dynaflow_amd.manager import DynaFlowManager
+    from dynaflow_amd.mlp import SwiGLUMLP
+
+    tokens, hidden, inter = 512, 512, 1408
+    cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", 2, InductorConfig(enabled=True),
+                         CUDAGraphConfig(enabled=True, capture_sizes=[256, 512]),
+                         {"min_nano_split_tokens": 1, "num_nano_batches": 2, "dump_graph": False, "max_tokens": 1024})
+    x, wg, wu, wd = mlp.make_inputs(tokens, hidden, inter, torch.bfloat16)
+    model = SwiGLUMLP(hidden, inter, dtype=torch.bfloat16, device="cuda")
+    with torch.no_grad():
+        model.gate_proj.weight.copy_(wg)
+        model.up_proj.weight.copy_(wu)
+        model.down_proj.weight.copy_(wd)
+    manager = DynaFlowManager()
+    torch._dynamo.reset()
+    xg = x.cuda()
+    torch._dynamo.mark_dynamic(xg, 0)
+    compiled = torch.compile(model, backend=make_backend(manager, cfg), fullgraph=True)
+    with torch.no_grad():
+        manager.prepare(tokens, [tokens])
+        compiled(xg)                                   # trace
+        eager = compiled_eager = None
+        manager.prepare(tokens, [tokens])
+        eager = compiled(xg).clone()                   # scheduled, no graphs
+        # dry-run at the nano-batch size: captures (256, 0) and (256, 1) for both sub-graphs
+        half = xg[:256].contiguous()
+        manager.prepare(256, [256], is_dryrun=True, use_cudagraph=True)
+        dry = compiled(half)
+        torch.cuda.synchronize()
+        assert torch.equal(dry, eager[:256])
+        # scheduled forward replaying the captured graphs
+        split = SplitConfig(2, [256, 256], [0, 256, 512], [256, 256], [256, 256], [0, 256, 512], False, True)
+        for _ in range(3):
+            manager.override_split_config(split)
+            y = compiled(xg)
+            torch.cuda.synchronize()
+            assert torch.equal(y, eager)
+            torch.randn(256, 256, device="cuda").sum().item()
+        # new values flow through the static buffers
+        xg2 = torch.randn_like(xg)
+        manager.prepare(tokens, [tokens])
+        want = compiled(xg2).clone()
+        manager.override_split_config(split)
+        assert torch.equal(compiled(xg2), want)
+        # a size that was never captured cannot be replayed
+        bad = SplitConfig(2, [128, 384], [0, 128, 512], [128, 384], [128, 384], [0, 128, 512], False, True)
+        manager.override_split_config(bad)
+        with pytest.raises(AssertionError):
+            compiled(xg)
+    for name in ("submod_0", "submod_1"):
+        wrapper = manager.graph_module.__dict__[name].callable_dynamic
+        assert sorted(k[:2] for k in wrapper._entries) == [(256, 0), (256, 1)]
