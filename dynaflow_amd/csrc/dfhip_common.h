@@ -60,3 +60,18 @@ DFHIP_DEVICE int remap_xcd(int pid, int total) {
   const int start = xcd * base + (xcd < rem ? xcd : rem);
   return start + local;
 }
+
+// ---- hand-ordered memory operations of the LDS-DMA GEMM kernels ------------------------------
+// One LDS-DMA instruction: 64 lanes x 16 bytes from per-lane global addresses to
+// LDS[lds_addr + 16*lane].  The compiler does not see the memory effect; ordering is kept by
+// hand with wait_vmcnt / workgroup_barrier.
+DFHIP_DEVICE void dma16(uint32_t lds_addr, const void* g) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(g)
+               : "memory", "m0");
+}
+template <int N>
+DFHIP_DEVICE void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+DFHIP_DEVICE void workgroup_barrier() { asm volatile("s_barrier" ::: "memory"); }
+#define DFHIP_PIN __builtin_amdgcn_sched_barrier(0)

@@ -1,13 +1,17 @@
 // fp8 (OCP e4m3fn) path: per-tensor dynamic quantisation, SiLU*mul with amax,
 // and the fp8 GEMM  C = bf16(a_scale * w_scale[n] * A[M,K] * W[N,K]^T).
 //
-// The GEMM has the byte geometry of the bf16 one (a K slab row is 128 bytes,
-// here 128 fp8 values): 16-byte global loads staged through registers into two
-// padded LDS buffers, one barrier per slab.  It multiplies with
-// v_mfma_scale_f32_32x32x64_f8f6f4 (scale exponents fixed at 2^0), which
-// retires 64 k per instruction - twice the bf16 rate.  A lane feeds 32
-// consecutive bytes of one row; both operands use the same lane->k mapping, so
-// the contraction is exact whatever order the hardware walks those bytes in.
+// The GEMMs have the byte geometry of the bf16 ones (a K slab row is 128 bytes, here
+// 128 fp8 values) and multiply with v_mfma_scale_f32_32x32x64_f8f6f4 (scale exponents
+// fixed at 2^0), which retires 64 k per instruction - twice the bf16 rate.  A lane
+// feeds 32 consecutive bytes of one row; both operands use the same lane->k mapping,
+// so the contraction is exact whatever order the hardware walks those bytes in.
+//
+// gemm_fp8_ring_kernel  256x256 tile, the LDS-DMA ring / pinned-schedule design of the
+//                       bf16 ring kernel: five 32 KiB LDS units, 1.5 slabs in flight,
+//                       XOR-swizzled 128-byte rows, one LDS read or DMA issue behind every
+//                       MFMA, barrier between the two k-steps of a slab, staged epilogue.
+// gemm_fp8_nt_kernel    register-staged double buffer for small shapes.
 #include "dfhip_common.h"
 
 namespace {
@@ -233,6 +237,174 @@ gemm_fp8_nt_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
   }
 }
 
+
+// ------------------------------------------------------------------ fp8 ring kernel
+constexpr int F8_UNIT = 32768, F8_NUNITS = 5, F8_RING_LDS = F8_UNIT * F8_NUNITS;
+constexpr int F8_GROUP_M = 4, F8_EROW = 272;
+
+__global__ void __launch_bounds__(256)
+gemm_fp8_ring_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, uint16_t* __restrict__ C,
+                     const float* __restrict__ a_scale, const float* __restrict__ w_scale, int M, int N, int K,
+                     int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave & 1, wave_n = wave >> 1;
+
+  const int tile = remap_xcd(blockIdx.x, tiles_m * tiles_n);
+  const int per_panel = F8_GROUP_M * tiles_n;
+  const int first_m = (tile / per_panel) * F8_GROUP_M;
+  const int rows_in_panel = (tiles_m - first_m) < F8_GROUP_M ? (tiles_m - first_m) : F8_GROUP_M;
+  const int in_panel = tile % per_panel;
+  const int m0 = (first_m + in_panel % rows_in_panel) * 256;
+  const int n0 = (in_panel / rows_in_panel) * 256;
+  const int KT = K / FBK;
+
+  const uint8_t* a_src[8];
+  const uint8_t* w_src[8];
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    const int row = (wave * 8 + t) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    int ar = m0 + row; ar = ar < M ? ar : M - 1;
+    int wr = n0 + row; wr = wr < N ? wr : N - 1;
+    a_src[t] = A + (int64_t)ar * lda + chunk * 16;
+    w_src[t] = W + (int64_t)wr * ldw + chunk * 16;
+  }
+  const uint32_t wave_lds = wave * 8 * 1024;
+  auto dma_a = [&](int t, int slab, int unit) {
+    const int s = slab < KT ? slab : KT - 1;
+    dma16(unit * F8_UNIT + wave_lds + t * 1024, a_src[t] + (int64_t)s * FBK);
+  };
+  auto dma_w = [&](int t, int slab, int unit) {
+    const int s = slab < KT ? slab : KT - 1;
+    dma16(unit * F8_UNIT + wave_lds + t * 1024, w_src[t] + (int64_t)s * FBK);
+  };
+
+  // a fragment is 32 bytes = chunks c and c^1 with c = 4*ks + 2*(lane/32), swizzled by (row/2)%8
+  const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
+  int koff[2][2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    koff[ks][0] = ((4 * ks + 2 * fhalf) ^ fswz) * 16;
+    koff[ks][1] = ((4 * ks + 2 * fhalf + 1) ^ fswz) * 16;
+  }
+  const int a_lane = (wave_m * 128 + frow) * 128, w_lane = (wave_n * 128 + frow) * 128;
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_a(t, 0, 0);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_w(t, 0, 1);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_a(t, 1, 2);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_w(t, 1, 3);
+  wait_vmcnt<16>();
+  workgroup_barrier();
+
+  u32x4 fa[2][4][2], fw[2][4][2];   // [slot][block][low/high 16 bytes]
+  auto read_half = [&](int r, int ks, int slot, int unit_a, int unit_w) {  // r 0..7: A, 8..15: W
+    const int blk = (r & 7) >> 1, part = r & 1;
+    if (r < 8)
+      fa[slot][blk][part] = *reinterpret_cast<const u32x4*>(smem + unit_a * F8_UNIT + a_lane + koff[ks][part] + blk * 4096);
+    else
+      fw[slot][blk][part] = *reinterpret_cast<const u32x4*>(smem + unit_w * F8_UNIT + w_lane + koff[ks][part] + blk * 4096);
+  };
+  auto mfma = [&](int q, int slot) {
+    const int i = q >> 2, j = q & 3;
+    const i32x8 av = {(int)fa[slot][i][0][0], (int)fa[slot][i][0][1], (int)fa[slot][i][0][2], (int)fa[slot][i][0][3],
+                      (int)fa[slot][i][1][0], (int)fa[slot][i][1][1], (int)fa[slot][i][1][2], (int)fa[slot][i][1][3]};
+    const i32x8 wv = {(int)fw[slot][j][0][0], (int)fw[slot][j][0][1], (int)fw[slot][j][0][2], (int)fw[slot][j][0][3],
+                      (int)fw[slot][j][1][0], (int)fw[slot][j][1][1], (int)fw[slot][j][1][2], (int)fw[slot][j][1][3]};
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wv, av, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+  };
+
+  int ua = 0, uw = 1, ia = 4, iw = 0;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) read_half(r, 0, 0, ua, uw);
+  for (int kt = 0; kt < KT; ++kt) {
+    // k-step 0: one fragment half of step 1 behind every MFMA, DMA of A(kt+2) behind every other one
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      mfma(q, 0);
+      read_half(q, 1, 1, ua, uw);
+      if (q & 1) dma_a(q >> 1, kt + 2, ia);
+      DFHIP_PIN;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    wait_vmcnt<8>();
+    workgroup_barrier();
+    int na = ua + 2; if (na >= F8_NUNITS) na -= F8_NUNITS;
+    int nw = uw + 2; if (nw >= F8_NUNITS) nw -= F8_NUNITS;
+    // k-step 1: DMA of W(kt+2) and the fragments of slab kt+1, step 0
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      mfma(q, 1);
+      if (!(q & 1)) dma_w(q >> 1, kt + 2, iw);
+      read_half(q, 0, 0, na, nw);
+      DFHIP_PIN;
+    }
+    ua = na; uw = nw;
+    ia += 2; if (ia >= F8_NUNITS) ia -= F8_NUNITS;
+    iw += 2; if (iw >= F8_NUNITS) iw -= F8_NUNITS;
+  }
+  wait_vmcnt<0>();
+  workgroup_barrier();
+
+  // scale, round to bf16, park the wave's 128x128 block in LDS, store whole 256-byte row pieces
+  const float sa = a_scale[0];
+  uint8_t* park = smem + wave * (128 * F8_EROW);
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      int n = n0 + wave_n * 128 + j * 32 + g * 8 + fhalf * 4;
+      n = n < N ? n : N - 4;   // columns past the edge are never stored; keep the scale load in bounds
+      const f32x4 ws = *reinterpret_cast<const f32x4*>(w_scale + n);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        u32x2 v;
+        v[0] = pack2_bf16(acc[i][j][4 * g + 0] * (sa * ws[0]), acc[i][j][4 * g + 1] * (sa * ws[1]));
+        v[1] = pack2_bf16(acc[i][j][4 * g + 2] * (sa * ws[2]), acc[i][j][4 * g + 3] * (sa * ws[3]));
+        *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * F8_EROW + (j * 32 + g * 8 + fhalf * 4) * 2) = v;
+      }
+    }
+  DFHIP_PIN;
+  const int m_base = m0 + wave_m * 128, n_base = n0 + wave_n * 128;
+#pragma unroll 4
+  for (int p = 0; p < 32; ++p) {
+    const int id = p * 64 + lane;
+    const int row = id >> 4, c = id & 15;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * F8_EROW + c * 16);
+    const int m = m_base + row, n = n_base + c * 8;
+    if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+  }
+}
+
+int launch_fp8_ring(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
+                    const float* a_scale, const float* w_scale, int M, int N, int K, hipStream_t stream) {
+  static bool lds_opted_in = false;
+  if (!lds_opted_in) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fp8_ring_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, F8_RING_LDS) != hipSuccess)
+      return DFHIP_ERR_LAUNCH;
+    lds_opted_in = true;
+  }
+  const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+  hipLaunchKernelGGL(gemm_fp8_ring_kernel, dim3(tiles_m * tiles_n), dim3(256), F8_RING_LDS, stream,
+                     static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(W), static_cast<uint16_t*>(C),
+                     a_scale, w_scale, M, N, K, lda, ldw, ldc, tiles_m, tiles_n);
+  return dfhip_check_launch();
+}
+
 template <int BM, int BN>
 int launch_fp8(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, const float* a_scale,
                const float* w_scale, int M, int N, int K, hipStream_t stream) {
@@ -317,6 +489,7 @@ extern "C" int dfhip_gemm_fp8_nt(const void* A, int64_t lda, const void* W, int6
     return DFHIP_ERR_BAD_ALIGNMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-  if (M > 128 && big_tiles >= 192) return launch_fp8<256, 256>(A, lda, W, ldw, C, ldc, a_scale, w_scale, M, N, K, s);
+  if (M > 128 && N > 128 && big_tiles >= 32)
+    return launch_fp8_ring(A, lda, W, ldw, C, ldc, a_scale, w_scale, M, N, K, s);
   return launch_fp8<128, 128>(A, lda, W, ldw, C, ldc, a_scale, w_scale, M, N, K, s);
 }

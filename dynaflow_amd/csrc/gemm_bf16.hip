@@ -201,19 +201,6 @@ constexpr int UNIT = 32768, NUNITS = 5, RING_LDS = UNIT * NUNITS;
 constexpr int GROUP_M = 4;   // tiles of one XCD are walked in panels of GROUP_M tile rows
 constexpr int EROW = 272;    // padded row of the epilogue staging area (bytes)
 
-// One LDS-DMA instruction: 64 lanes x 16 bytes from per-lane global addresses to
-// LDS[lds_addr + 16*lane].  The compiler does not see the memory effect; ordering
-// is kept by hand with s_waitcnt vmcnt / s_barrier below.
-DFHIP_DEVICE void dma16(uint32_t lds_addr, const void* g) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(g)
-               : "memory", "m0");
-}
-template <int N>
-DFHIP_DEVICE void wait_vmcnt() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-DFHIP_DEVICE void workgroup_barrier() { asm volatile("s_barrier" ::: "memory"); }
-
 // 16-byte store / load that is coherent across the XCDs (sc1: written through to, and read
 // from, the memory side instead of the XCD-private L2).  Used for split-K partial blocks so
 // that no L2-wide write-back or invalidate is needed to hand them from one XCD to another.
@@ -228,7 +215,6 @@ DFHIP_DEVICE f32x4 load_f32x4_device_coherent(const f32x4* p) {
 // The loads above are invisible to the compiler's own wait-count bookkeeping: a value may only
 // be used after this, which ties the wait to the register so that the use cannot move above it.
 DFHIP_DEVICE void wait_loaded(f32x4& v) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(v)::"memory"); }
-#define DFHIP_PIN __builtin_amdgcn_sched_barrier(0)
 
 __global__ void __launch_bounds__(RTHREADS)
 gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, uint16_t* __restrict__ C,

@@ -199,7 +199,8 @@ def test_silu_mul_quant_fp8(ops):
     assert bool(((got == want_q) | ((got & 0x7F == 0) & (want_q & 0x7F == 0))).all())
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 8, 128), (65, 72, 256), (300, 264, 384), (512, 1024, 1024)])
+@pytest.mark.parametrize("M,N,K", [(1, 8, 128), (65, 72, 256), (300, 264, 384), (512, 1024, 1024),
+                                   (2048, 1024, 1024), (1100, 2056, 384), (1536, 1536, 128)])
 def test_gemm_fp8_against_dequantised_fp32(ops, M, N, K):
     x = randn((M, K), 20).bfloat16()
     w = randn((N, K), 21, 0.02).bfloat16()
