@@ -49,6 +49,9 @@ def parse_args():
     p.add_argument("--kernels-only", action="store_true",
                    help="run only the single-kernel timing loops plus a 256 MiB device copy (used to calibrate "
                         "FETCH_SIZE / WRITE_SIZE under rocprofv3 --pmc); prints the kernel figures as JSON")
+    p.add_argument("--fp8", action="store_true",
+                   help="measure the fp8 70B-shaped MLP layer (x[8192,8192], I=28672, 4 nano-batches of 2048) "
+                        "instead of the headline bf16 configuration")
     return p.parse_args()
 
 
@@ -129,6 +132,66 @@ def single_kernels(torch, ops, x, weights, iters, calibration_copy=False):
     return out
 
 
+def fp8_config(torch, steps, warmup):
+    """fp8 70B-shaped layer: x[8192,8192] bf16 quantised per tensor inside the graph, weights e4m3 with
+    per-output-channel scales, 4 nano-batches of 2048 through the manager on two streams."""
+    from dynaflow_amd.backend import make_backend
+    from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
+    from dynaflow_amd.fp8_mlp import Fp8SwiGLU
+    from dynaflow_amd.manager import DynaFlowManager
+
+    tokens, hidden, inter, splits = 8192, 8192, 28672, 4
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(tokens, hidden, generator=gen, device="cuda", dtype=torch.float32).bfloat16()
+    parts = []
+    for shape in ((inter, hidden), (inter, hidden), (hidden, inter)):
+        w = (torch.randn(shape, generator=gen, device="cuda", dtype=torch.float32) * 0.02).bfloat16()
+        parts.append(w)
+    layer = Fp8SwiGLU.from_weights(*parts)
+    del parts
+    results = {}
+    for name, knobs in (("serialized", {"serialize": True}), ("overlapped", {"whole_graph": True})):
+        extra = {"min_nano_split_tokens": 64, "num_nano_batches": splits, "dump_graph": False}
+        extra.update(knobs)
+        cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", splits, InductorConfig(enabled=True),
+                             CUDAGraphConfig(enabled=False, capture_sizes=[tokens]), extra)
+        manager = DynaFlowManager()
+        torch._dynamo.reset()
+        torch._dynamo.mark_dynamic(x, 0)
+        compiled = torch.compile(layer, backend=make_backend(manager, cfg), fullgraph=True)
+        with torch.no_grad():
+            manager.prepare(tokens, [tokens])
+            compiled(x)
+
+            def step(use_graph):
+                manager.prepare(tokens, [tokens], use_cudagraph=use_graph)
+                return compiled(x)
+
+            modes = (("eager", False),) if name == "serialized" else (("eager", False), ("graph", True))
+            for mode, use_graph in modes:
+                for _ in range(warmup):
+                    step(use_graph)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    step(use_graph)
+                torch.cuda.synchronize()
+                results[f"{name}_{mode}_ms"] = (time.perf_counter() - t0) * 1e3 / steps
+    flops = 6.0 * tokens * hidden * inter
+    best = results["overlapped_graph_ms"]
+    return {
+        "metric": "fp8 MLP-layer tokens/s, 70B-shape e4m3, 1 MI355X",
+        "value": tokens / (best * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": best, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3",
+        "data": "synthetic",
+        "config": {"workload": "fp8 70B-shaped SwiGLU MLP layer, x[8192,8192], I=28672, 4 nano-batches of 2048, "
+                               "per-tensor activation / per-channel weight scales, bf16 output"},
+        "timings": results,
+        "layer": {"tflops": flops / (best * 1e-3) / 1e12, "frac_of_fp8_mfma_peak": flops / (best * 1e-3) / 1e12 / 5000.0},
+        "overlap_speedup": results["serialized_eager_ms"] / best,
+    }
+
+
 def cpu_baseline(torch):
     """The schedule restated with eager PyTorch on the host cores, on a bounded sample."""
     from oracle import mlp as oracle_mlp
@@ -185,6 +248,9 @@ def main() -> int:
 
     _cabi.load()
     info = _cabi.device_info(0)
+    if args.fp8:
+        print(json.dumps(fp8_config(torch, max(5, args.steps // 5), max(3, args.warmup // 5))))
+        return 0
     x_cpu, wg, wu, wd = oracle_mlp.make_inputs(TOKENS, HIDDEN, INTER, torch.bfloat16, prenorm=True)
     x = x_cpu.cuda()
     weights = (wg.cuda(), wu.cuda(), wd.cuda())

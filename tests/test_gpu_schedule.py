@@ -253,3 +253,55 @@ def test_piecewise_graphs_capture_in_dryrun_and_replay():
     for name in ("submod_0", "submod_1"):
         wrapper = manager.graph_module.__dict__[name].callable_dynamic
         assert sorted(k[:2] for k in wrapper._entries) == [(256, 0), (256, 1)]
+
+
+def test_fp8_config_full_size_properties():
+    """fp8 70B-shaped layer at full size (x[8192,8192], I=28672, 4 x 2048).  The CPU oracle cannot cover
+    this size in test time; the kernels are pinned on small shapes, here the schedule is: (1) the scheduled
+    two-stream run equals the nano-batches issued one after the other bit for bit, (2) two runs agree,
+    (3) sampled rows agree with an fp32 evaluation of the same quantised operands done with torch on the GPU."""
+    from dynaflow_amd.backend import make_backend
+    from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
+    from dynaflow_amd.fp8_mlp import Fp8SwiGLU
+    from dynaflow_amd.manager import DynaFlowManager
+
+    tokens, hidden, inter = 8192, 8192, 28672
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(tokens, hidden, generator=gen, device="cuda").bfloat16()
+    ws = [(torch.randn(s, generator=gen, device="cuda") * 0.02).bfloat16() for s in ((inter, hidden), (inter, hidden), (hidden, inter))]
+    layer = Fp8SwiGLU.from_weights(*ws)
+    del ws
+    cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", 4, InductorConfig(enabled=True),
+                         CUDAGraphConfig(enabled=False, capture_sizes=[tokens]),
+                         {"min_nano_split_tokens": 64, "num_nano_batches": 4, "dump_graph": False})
+    manager = DynaFlowManager()
+    torch._dynamo.reset()
+    torch._dynamo.mark_dynamic(x, 0)
+    compiled = torch.compile(layer, backend=make_backend(manager, cfg), fullgraph=True)
+    with torch.no_grad():
+        manager.prepare(tokens, [tokens])
+        compiled(x)
+        split = manager.prepare(tokens, [tokens])
+        y = compiled(x)
+        manager.prepare(tokens, [tokens])
+        y2 = compiled(x)
+        direct = layer.forward_schedule(x, split.split_indices)
+    torch.cuda.synchronize()
+    assert split.split_indices == [0, 2048, 4096, 6144, 8192]
+    assert torch.equal(y, y2) and torch.equal(y, direct)
+    # fp32 evaluation of nano-batch 0, rows 0..7, on the same e4m3 operands
+    from dynaflow_amd import ops
+    xb = x[:2048]
+    xq, xs = ops.quant_fp8(xb)
+    rows = slice(0, 8)
+    xd = xq[rows].float() * xs
+    g = (xd @ (layer.w_gate_q.float() * layer.w_gate_s[:, None]).t()).bfloat16()
+    u = (xd @ (layer.w_up_q.float() * layer.w_up_s[:, None]).t()).bfloat16()
+    # the re-quantisation scale of the SiLU*mul output needs the whole nano-batch: take it from the kernels
+    gate_full = ops.linear_fp8(xq, layer.w_gate_q, xs, layer.w_gate_s)
+    up_full = ops.linear_fp8(xq, layer.w_up_q, xs, layer.w_up_s)
+    aq, a_s = ops.silu_mul_quant_fp8(gate_full, up_full)
+    assert rel_err(gate_full[rows].float(), g.float()) < 2 ** -6
+    assert rel_err(up_full[rows].float(), u.float()) < 2 ** -6
+    want = (aq[rows].float() * a_s) @ (layer.w_down_q.float() * layer.w_down_s[:, None]).t()
+    assert rel_err(y[rows].float(), want) < TOL["fp8"]
