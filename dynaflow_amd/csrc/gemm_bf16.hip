@@ -216,10 +216,19 @@ DFHIP_DEVICE f32x4 load_f32x4_device_coherent(const f32x4* p) {
 // be used after this, which ties the wait to the register so that the use cannot move above it.
 DFHIP_DEVICE void wait_loaded(f32x4& v) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(v)::"memory"); }
 
+// FUSED = false: C[M,N] = A W^T.
+// FUSED = true : C[M,N] = silu(A W^T) * (A W2^T) with W = gate weight, W2 = up weight, N = the
+//   intermediate size.  A tile is 256 rows x 128 columns; its "W half" holds 128 gate rows and 128 up
+//   rows arranged so that every wave owns gate AND up accumulators of the same 128x64 block (MFMA
+//   blocks j = 0,1 are gate, j = 2,3 are up): the SiLU*mul happens in registers, in fp32, on the
+//   unrounded projections, and only the product is written.
+template <bool FUSED>
 __global__ void __launch_bounds__(RTHREADS)
-gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, uint16_t* __restrict__ C,
+gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
+                      const uint16_t* __restrict__ W2, uint16_t* __restrict__ C,
                       int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n,
                       int split_k, float* __restrict__ partials, int* __restrict__ arrivals) {
+  constexpr int TILE_N = FUSED ? 128 : RBN;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -235,7 +244,7 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   const int rows_in_panel = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
   const int in_panel = tile % per_panel;
   const int m0 = (first_m + in_panel % rows_in_panel) * RBM;
-  const int n0 = (in_panel / rows_in_panel) * RBN;
+  const int n0 = (in_panel / rows_in_panel) * TILE_N;
   // this workgroup multiplies slabs [slab0, slab0 + KT) of the K / 64 slabs
   const int slabs_total = K / BK;
   const int slab0 = (int)((int64_t)slabs_total * part / split_k);
@@ -250,9 +259,17 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
     const int row = (wave * 8 + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     int ar = m0 + row; ar = ar < M ? ar : M - 1;   // rows past the edge re-read the last row; never stored
-    int wr = n0 + row; wr = wr < N ? wr : N - 1;
     a_src[t] = reinterpret_cast<const uint8_t*>(A + (int64_t)ar * lda + chunk * 8);
-    w_src[t] = reinterpret_cast<const uint8_t*>(W + (int64_t)wr * ldw + chunk * 8);
+    if (FUSED) {
+      // LDS W row r: 64-row block r/64 = 2*wave_n + (0: gate, 1: up); column wave_n*64 + r%64 of the tile
+      const int block = row >> 6;
+      int wr = n0 + (block >> 1) * 64 + (row & 63); wr = wr < N ? wr : N - 1;
+      const uint16_t* base = (block & 1) ? W2 : W;
+      w_src[t] = reinterpret_cast<const uint8_t*>(base + (int64_t)wr * ldw + chunk * 8);
+    } else {
+      int wr = n0 + row; wr = wr < N ? wr : N - 1;
+      w_src[t] = reinterpret_cast<const uint8_t*>(W + (int64_t)wr * ldw + chunk * 8);
+    }
   }
   const uint32_t wave_lds = wave * 8 * 1024;
   auto dma_a = [&](int t, int slab, int unit) {
@@ -348,7 +365,7 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   wait_vmcnt<0>();      // the padding halves issued by the last iterations
   workgroup_barrier();  // other waves may still be reading fragments where this wave parks its block
 
-  if (split_k > 1) {
+  if (!FUSED && split_k > 1) {
     // Every part leaves its fp32 block in `partials` and takes a ticket; the part that draws the
     // last ticket adds all parts up in part order (so the sum does not depend on who came last)
     // and writes the tile.  Nobody waits for anybody.
@@ -400,6 +417,40 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
     }
   }
 
+  if (FUSED) {
+    // silu(gate) * up in registers, then park 128 rows x 64 columns per wave (144-byte rows)
+    constexpr int FROW_BYTES = 144;
+    uint8_t* park = smem + wave * (128 * FROW_BYTES);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          float p[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float gt = acc[i][j][4 * g + e];
+            p[e] = (gt / (1.0f + expf(-gt))) * acc[i][j + 2][4 * g + e];
+          }
+          u32x2 v;
+          v[0] = pack2_bf16(p[0], p[1]);
+          v[1] = pack2_bf16(p[2], p[3]);
+          *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * FROW_BYTES + (j * 32 + g * 8 + fhalf * 4) * 2) = v;
+        }
+    DFHIP_PIN;
+    const int m_base = m0 + wave_m * 128, n_base = n0 + wave_n * 64;
+#pragma unroll 4
+    for (int p = 0; p < 16; ++p) {
+      const int id = p * 64 + lane;
+      const int row = id >> 3, c = id & 7;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * FROW_BYTES + c * 16);
+      const int m = m_base + row, n = n_base + c * 8;
+      if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+    }
+    return;
+  }
+
   uint8_t* park = smem + wave * (128 * EROW);
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -424,16 +475,19 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   }
 }
 
-int launch_ring(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K,
-                int split_k, void* workspace, hipStream_t stream) {
-  static bool lds_opted_in = false;
+template <bool FUSED>
+int launch_ring(const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw, void* C, int64_t ldc, int M,
+                int N, int K, int split_k, void* workspace, hipStream_t stream) {
+  auto kernel = gemm_bf16_ring_kernel<FUSED>;
+  static bool lds_opted_in = false;   // one flag per instantiation
   if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_ring_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, RING_LDS) != hipSuccess)
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            RING_LDS) != hipSuccess)
       return DFHIP_ERR_LAUNCH;
     lds_opted_in = true;
   }
-  const int tiles_m = (M + RBM - 1) / RBM, tiles_n = (N + RBN - 1) / RBN;
+  const int tiles_m = (M + RBM - 1) / RBM;
+  const int tiles_n = FUSED ? (N + 127) / 128 : (N + RBN - 1) / RBN;
   // workspace layout: [tiles] arrival counters (padded to 256 bytes), then [tiles][split_k] fp32 blocks
   int* arrivals = static_cast<int*>(workspace);
   float* partials = nullptr;
@@ -441,9 +495,10 @@ int launch_ring(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
     const size_t counter_bytes = (((size_t)tiles_m * tiles_n * sizeof(int)) + 255) & ~(size_t)255;
     partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + counter_bytes);
   }
-  hipLaunchKernelGGL(gemm_bf16_ring_kernel, dim3(tiles_m * tiles_n * split_k), dim3(RTHREADS), RING_LDS, stream,
-                     static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W), static_cast<uint16_t*>(C), M, N,
-                     K, lda, ldw, ldc, tiles_m, tiles_n, split_k, partials, arrivals);
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * split_k), dim3(RTHREADS), RING_LDS, stream,
+                     static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W),
+                     static_cast<const uint16_t*>(W2), static_cast<uint16_t*>(C), M, N, K, lda, ldw, ldc, tiles_m,
+                     tiles_n, split_k, partials, arrivals);
   return dfhip_check_launch();
 }
 
@@ -485,7 +540,7 @@ extern "C" int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void
   if (int rc = check_args(A, lda, W, ldw, C, ldc, M, N, K)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (variant) {
-    case 0: return launch_ring(A, lda, W, ldw, C, ldc, M, N, K, 1, nullptr, s);
+    case 0: return launch_ring<false>(A, lda, W, nullptr, ldw, C, ldc, M, N, K, 1, nullptr, s);
     case 4: return launch<256, 256, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 1: return launch<256, 256, 2, 4>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 2: return launch<128, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
@@ -537,5 +592,16 @@ extern "C" int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void*
     if (!dfhip_aligned16(workspace)) return DFHIP_ERR_BAD_ALIGNMENT;
     if (workspace_bytes < dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k)) return DFHIP_ERR_BAD_ARGUMENT;
   }
-  return launch_ring(A, lda, W, ldw, C, ldc, M, N, K, split_k, workspace, static_cast<hipStream_t>(stream));
+  return launch_ring<false>(A, lda, W, nullptr, ldw, C, ldc, M, N, K, split_k, workspace,
+                            static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dfhip_gemm_bf16_gate_up_silu(const void* A, int64_t lda, const void* W_gate, const void* W_up,
+                                            int64_t ldw, void* Out, int64_t ldo, int M, int I, int K,
+                                            dfhip_stream_t stream) {
+  if (!W_up) return DFHIP_ERR_NULL_POINTER;
+  if (int rc = check_args(A, lda, W_gate, ldw, Out, ldo, M, I, K)) return rc;
+  if (!dfhip_aligned16(W_up)) return DFHIP_ERR_BAD_ALIGNMENT;
+  return launch_ring<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, 1, nullptr,
+                           static_cast<hipStream_t>(stream));
 }

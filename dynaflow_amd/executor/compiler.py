@@ -40,6 +40,7 @@ class SubgraphBackend:
         *,
         use_inductor: bool,
         use_cudagraph: bool,
+        lowering_options: dict | None = None,
     ) -> None:
         assert not use_inductor or inductor_config.enabled
         assert not use_cudagraph or cudagraph_config.enabled
@@ -55,6 +56,7 @@ class SubgraphBackend:
         self.callable_dynamic: Callable[..., Any] | None = None
         self.callables_per_size: dict[int, Callable[..., Any]] = {}
         self.lowering_stats: dict[str, int] = {}
+        self.lowering_options = dict(lowering_options or {})
 
     def compile(self, example_inputs: list[Any], runtime_shape: int | None = None) -> Callable[..., Any]:
         """Build the callable for the dynamic shape or for one fixed size."""
@@ -64,7 +66,7 @@ class SubgraphBackend:
         if self.use_inductor:
             from dynaflow_amd.executor.hip_lowering import lower_to_hip
 
-            fn, self.lowering_stats = lower_to_hip(self.gm)
+            fn, self.lowering_stats = lower_to_hip(self.gm, **self.lowering_options)
         if self.use_cudagraph:
             fn = CUDAGraphWrapper(fn, self.cudagraph_config)
         return fn
@@ -132,6 +134,7 @@ class SubgraphCompiler(fx.Interpreter):
             self.config.cudagraph_config,
             use_inductor=target in self.inductor_compile_targets,
             use_cudagraph=target in self.cudagraph_targets,
+            lowering_options={"fuse_silu_epilogue": bool(self.config.knob("fuse_silu_epilogue", False))},
         )
         backend.callable_dynamic = backend.compile(list(args))
         self.module.__dict__[target] = backend

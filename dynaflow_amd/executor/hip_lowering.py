@@ -7,6 +7,10 @@ it deep-copies the sub-``GraphModule`` and replaces
 * ``linear(x, w)`` (no bias, bf16 or fp32)            -> ``dynaflow_hip.linear``
 * ``mul(silu(g), u)`` / ``mul(u, silu(g))``           -> ``dynaflow_hip.silu_mul``
 
+With ``fuse_silu_epilogue`` a third rewrite follows: a ``silu_mul`` whose gate and up
+inputs are two bf16 ``linear`` nodes of the same activation becomes one
+``dynaflow_hip.gate_up_silu(x, w_gate, w_up)`` - the SiLU*mul as the GEMM's epilogue.
+
 Everything else stays as traced and keeps running on PyTorch's own ROCm
 kernels.  The pass only decides by what tracing recorded (``example_value``
 dtypes and static trailing dimensions); token counts stay symbolic.
@@ -74,7 +78,7 @@ def _silu_mul_supported(g: Any) -> bool:
     return False
 
 
-def lower_to_hip(gm: fx.GraphModule) -> tuple[fx.GraphModule, dict[str, int]]:
+def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False) -> tuple[fx.GraphModule, dict[str, int]]:
     """Return a lowered deep copy of ``gm`` and a count of each rewrite."""
     # registering the operators is a side effect of importing them
     from dynaflow_amd import ops
@@ -82,6 +86,8 @@ def lower_to_hip(gm: fx.GraphModule) -> tuple[fx.GraphModule, dict[str, int]]:
     lowered = copy.deepcopy(gm)
     graph = lowered.graph
     stats = {"linear": 0, "silu_mul": 0}
+    if fuse_silu_epilogue:
+        stats["gate_up_silu"] = 0
 
     for node in list(graph.nodes):
         name = _target_name(node)
@@ -124,6 +130,31 @@ def lower_to_hip(gm: fx.GraphModule) -> tuple[fx.GraphModule, dict[str, int]]:
             graph.erase_node(silu)
             stats["silu_mul"] += 1
             break
+
+    if fuse_silu_epilogue:
+        for node in list(graph.nodes):
+            if node.op != "call_function" or node.target is not ops.silu_mul:
+                continue
+            gate, up = node.args[0], node.args[1]
+            if not (isinstance(gate, fx.Node) and isinstance(up, fx.Node)):
+                continue
+            if gate.target is not ops.linear or up.target is not ops.linear:
+                continue
+            if gate.args[0] is not up.args[0] or len(gate.users) != 1 or len(up.users) != 1:
+                continue
+            eg = _example(gate)
+            if not isinstance(eg, torch.Tensor) or eg.dtype != torch.bfloat16:
+                continue
+            with graph.inserting_before(node):
+                new = graph.call_function(ops.gate_up_silu, (gate.args[0], gate.args[1], up.args[1]))
+            new.meta = dict(node.meta)
+            node.replace_all_uses_with(new)
+            graph.erase_node(node)
+            graph.erase_node(gate)
+            graph.erase_node(up)
+            stats["gate_up_silu"] += 1
+            stats["linear"] -= 2
+            stats["silu_mul"] -= 1
 
     graph.lint()
     lowered.recompile()

@@ -31,6 +31,7 @@ _lib = torch.library.Library("dynaflow_hip", "DEF")
 _lib.define("linear(Tensor x, Tensor weight) -> Tensor")
 _lib.define("linear_variant(Tensor x, Tensor weight, int variant) -> Tensor")
 _lib.define("silu_mul(Tensor gate, Tensor up, bool round_silu=False) -> Tensor")
+_lib.define("gate_up_silu(Tensor x, Tensor w_gate, Tensor w_up) -> Tensor")
 _lib.define("rms_norm(Tensor x, Tensor weight, float eps) -> Tensor")
 _lib.define("add_rms_norm(Tensor x, Tensor residual, Tensor weight, float eps) -> (Tensor, Tensor)")
 _lib.define("transpose_weight(Tensor w) -> Tensor")
@@ -148,6 +149,36 @@ _lib.impl("linear", lambda x, w: _linear_impl(x, w), "CUDA")
 _lib.impl("linear_variant", lambda x, w, v: _linear_impl(x, w, v), "CUDA")
 torch.library.register_fake("dynaflow_hip::linear", _linear_fake, lib=_lib)
 torch.library.register_fake("dynaflow_hip::linear_variant", lambda x, w, v: _linear_fake(x, w), lib=_lib)
+
+
+# ------------------------------------------- gate/up projection + SiLU*mul epilogue
+def _gate_up_silu_impl(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor) -> torch.Tensor:
+    """``silu(x @ w_gate.T) * (x @ w_up.T)`` in one launch (bf16, weights in ``linear`` layout)."""
+    _require_device(x, w_gate, w_up)
+    lib = _cabi.load()
+    if x.dtype != torch.bfloat16 or w_gate.dtype != torch.bfloat16 or w_up.dtype != torch.bfloat16:
+        raise RuntimeError("gate_up_silu: bf16 only")
+    if w_gate.shape != w_up.shape or w_gate.dim() != 2 or x.shape[-1] != w_gate.shape[1]:
+        raise RuntimeError("gate_up_silu: shape mismatch")
+    a, M, K, lda = _rows(x)
+    wg, I, _, ldg = _rows(w_gate)
+    wu, _, _, ldu = _rows(w_up)
+    if ldg != ldu:
+        wg, wu = wg.contiguous(), wu.contiguous()
+        ldg = K
+    out = torch.empty((M, I), dtype=x.dtype, device=x.device)
+    if M > 0:
+        rc = lib.dfhip_gemm_bf16_gate_up_silu(
+            a.data_ptr(), lda, wg.data_ptr(), wu.data_ptr(), ldg, out.data_ptr(), I, M, I, K, _stream()
+        )
+        _cabi.check("dfhip_gemm_bf16_gate_up_silu", rc)
+    return out.view(*x.shape[:-1], I)
+
+
+_lib.impl("gate_up_silu", _gate_up_silu_impl, "CUDA")
+torch.library.register_fake(
+    "dynaflow_hip::gate_up_silu", lambda x, wg, wu: x.new_empty((*x.shape[:-1], wg.shape[0])), lib=_lib
+)
 
 
 # -------------------------------------------------------------- silu * mul
@@ -337,6 +368,7 @@ torch.library.register_fake(
 linear = torch.ops.dynaflow_hip.linear
 linear_variant = torch.ops.dynaflow_hip.linear_variant
 silu_mul = torch.ops.dynaflow_hip.silu_mul
+gate_up_silu = torch.ops.dynaflow_hip.gate_up_silu
 rms_norm = torch.ops.dynaflow_hip.rms_norm
 add_rms_norm = torch.ops.dynaflow_hip.add_rms_norm
 transpose_weight = torch.ops.dynaflow_hip.transpose_weight

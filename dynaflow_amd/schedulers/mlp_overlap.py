@@ -11,6 +11,11 @@ and the staggered order of ``StaggeredScheduler`` issues
 beside nano-batch i's SiLU*mul and down projection.  ``schedule="round_robin"``
 selects the NanoFlow order instead; both give the same per-stream order.
 
+With ``additional_config["fuse_silu_epilogue"]`` the cut moves in front of the down
+projection ({gate, up, silu, mul} | {down}) and the lowering turns the first sub-graph into
+one GEMM with the SiLU*mul as its epilogue; nano-batch i+1's fused GEMM then runs beside
+nano-batch i's down projection.
+
 Split policy: ``additional_config["num_nano_batches"]`` equal chunks (default
 ``max_num_splits``); with ``split_policy="balanced"`` the two-way balanced cut
 at a request boundary.
@@ -29,6 +34,7 @@ _SILU = r"silu(\.default)?"
 _MUL = r"mul(\.Tensor)?"
 
 TAIL_TAG = "tail"
+HEAD_TAG = "head"
 
 
 def mlp_split_rules() -> list[MatchingRule]:
@@ -44,6 +50,26 @@ def mlp_split_rules() -> list[MatchingRule]:
     ]
 
 
+def _follows_product(node_list, start_idx: int) -> bool:
+    """True for a ``linear`` whose input is the SiLU*mul product (the down projection)."""
+    node = node_list[start_idx]
+    producer = node.args[0] if node.args else None
+    name = getattr(getattr(producer, "target", None), "__name__", "")
+    return getattr(producer, "op", None) == "call_function" and name.split(".")[0] in ("mul", "silu_mul", "gate_up_silu")
+
+
+def mlp_split_rules_fused() -> list[MatchingRule]:
+    """Cut only in front of the down projection: {gate, up, silu, mul} | {down}, so that the
+    SiLU*mul can become the epilogue of the gate/up GEMM."""
+    return [MatchingRule(condition=Op(_LINEAR), hook=_follows_product)]
+
+
+def mlp_tag_rules_fused() -> dict[MatchingRule, set[str]]:
+    # inside the down-projection sub-graph the product is just an input, so the sub-graph that
+    # holds the product is the one that gets a tag (and the second stream)
+    return {MatchingRule(condition=Op(_MUL)): {HEAD_TAG}}
+
+
 def mlp_tag_rules() -> dict[MatchingRule, set[str]]:
     return {
         MatchingRule(condition=Op(_MUL)): {TAIL_TAG},
@@ -54,7 +80,10 @@ def mlp_tag_rules() -> dict[MatchingRule, set[str]]:
 
 class MLPOverlapScheduler(StaggeredScheduler):
     def __init__(self, config: DynaFlowConfig) -> None:
-        super().__init__(config, mlp_split_rules(), mlp_tag_rules(), side_tag=TAIL_TAG)
+        if config.knob("fuse_silu_epilogue", False):
+            super().__init__(config, mlp_split_rules_fused(), mlp_tag_rules_fused(), side_tag=HEAD_TAG)
+        else:
+            super().__init__(config, mlp_split_rules(), mlp_tag_rules(), side_tag=TAIL_TAG)
         self.policy_name = "mlp_overlap"
         self.num_nano_batches = config.knob("num_nano_batches", config.max_num_splits)
         self.split_policy = config.knob("split_policy", "equal")

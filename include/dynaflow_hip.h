@@ -105,6 +105,18 @@ int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void* W, int64_t
                               int64_t ldc, int M, int N, int K, int split_k, void* workspace,
                               size_t workspace_bytes, dfhip_stream_t stream);
 
+/* Gate and up projection with the SiLU*mul as the GEMM's epilogue:
+ *   Out[M,I] = bf16( silu(A W_gate^T) * (A W_up^T) )
+ * - the FX nodes linear, linear, silu, mul of the MLP in one launch.  Both
+ * weights [I,K] with the same leading dimension ldw.  The SiLU and the product
+ * are taken in fp32 on the unrounded projections (two separate kernels round
+ * gate and up to bf16 first), so results differ from dfhip_gemm_bf16_nt +
+ * dfhip_silu_mul_bf16 in the last bf16 bits.  Same shape rules as
+ * dfhip_gemm_bf16_nt with N = I. */
+int dfhip_gemm_bf16_gate_up_silu(const void* A, int64_t lda, const void* W_gate, const void* W_up,
+                                 int64_t ldw, void* Out, int64_t ldo, int M, int I, int K,
+                                 dfhip_stream_t stream);
+
 /* fp32 in / fp32 accumulate / fp32 out (the CPU-sized fp32 configuration).
  * Requires K % 4 == 0, 16-byte aligned pointers, lda/ldw % 4 == 0. */
 int dfhip_gemm_f32_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,

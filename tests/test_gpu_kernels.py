@@ -281,3 +281,21 @@ def test_down_projection_shape_uses_split_k_and_matches_unsplit(ops):
     rows = torch.tensor([0, 255, 256, 1023, 2047])
     want = a[rows].double().cpu() @ w.double().cpu().t()
     assert rel_err(split[rows].float(), want) < 2 ** -7
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 8, 64), (300, 264, 192), (257, 136, 128), (512, 1408, 512)])
+def test_gate_up_silu_fused_epilogue(ops, M, I, K):
+    """One launch for linear, linear, silu, mul: the epilogue takes SiLU and the product in fp32 on the
+    unrounded projections, so it is compared with an fp32 evaluation, one bf16 rounding apart."""
+    x = randn((M, K), 41).bfloat16()
+    wg = randn((I, K), 42, 0.05).bfloat16()
+    wu = randn((I, K), 43, 0.05).bfloat16()
+    g = x.double() @ wg.double().t()
+    want = (g / (1 + torch.exp(-g))) * (x.double() @ wu.double().t())
+    got = ops.gate_up_silu(x.cuda(), wg.cuda(), wu.cuda())
+    assert got.shape == (M, I) and got.dtype == torch.bfloat16
+    g32, w32 = got.float().cpu(), want.float()
+    assert bool(((g32 - w32).abs() <= 2 ** -7 * w32.abs() + 2e-4 * w32.abs().max()).all())
+    # and against the two-kernel path at the bf16 tolerance
+    two = ops.silu_mul(ops.linear(x.cuda(), wg.cuda()), ops.linear(x.cuda(), wu.cuda()), True)
+    assert rel_err(got.float(), two.float()) < TOL["bf16"]

@@ -305,3 +305,22 @@ def test_fp8_config_full_size_properties():
     assert rel_err(up_full[rows].float(), u.float()) < 2 ** -6
     want = (aq[rows].float() * a_s) @ (layer.w_down_q.float() * layer.w_down_s[:, None]).t()
     assert rel_err(y[rows].float(), want) < TOL["fp8"]
+
+
+def test_fused_silu_epilogue_schedule():
+    """fuse_silu_epilogue: {gate, up, silu, mul} becomes one GEMM with the SiLU*mul as epilogue, the cut
+    moves in front of the down projection; results stay within the bf16 tolerance of the oracle."""
+    from dynaflow_amd import ops
+
+    manager, compiled, xg, (x, wg, wu, wd) = build(1024, 1024, 2816, torch.bfloat16, fuse_silu_epilogue=True)
+    head = manager.graph_module.__dict__["submod_0"].callable_dynamic
+    tail = manager.graph_module.__dict__["submod_1"].callable_dynamic
+    assert [n.target for n in head.graph.nodes if n.op == "call_function"] == [ops.gate_up_silu]
+    assert [n.target for n in tail.graph.nodes if n.op == "call_function"] == [ops.linear]
+    y, split = run(manager, compiled, xg, 1024)
+    assert manager.engine.issue_trace == [("submod_0", 0), ("submod_1", 0), ("submod_0", 1), ("submod_1", 1)]
+    want = mlp.mlp_fp32_from(x, wg, wu, wd)
+    assert rel_err(y.float(), want) < TOL["bf16"]
+    unfused = build(1024, 1024, 2816, torch.bfloat16)
+    y0, _ = run(unfused[0], unfused[1], unfused[2], 1024)
+    assert rel_err(y.float(), y0.float()) < TOL["bf16"]
