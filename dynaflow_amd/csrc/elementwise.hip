@@ -1,14 +1,15 @@
 // HBM-bound kernels of the MLP path: SiLU*mul, RMSNorm, transpose, fill.
 //
-// All of them move 16 bytes per lane per access (global_load/store_dwordx4),
-// keep several loads in flight per lane before the first use, and do their
-// arithmetic in fp32 with a single rounding at the store.
+// All of them move 16 bytes per lane per access (global_load/store_dwordx4) from
+// many small workgroups and do their arithmetic in fp32 with a single rounding at
+// the store.
 #include "dfhip_common.h"
 
 namespace {
 
 constexpr int EW_THREADS = 256;
-constexpr int EW_UNROLL = 4;  // independent 16-byte groups per lane per array
+constexpr int EW_UNROLL = 1;  // 16-byte groups per lane per array: one is fastest here (6.5 vs 5.4 TB/s with four):
+                              // occupancy hides the latency better than a longer per-lane queue does
 
 DFHIP_DEVICE float silu_f32(float g) { return g / (1.0f + expf(-g)); }
 
