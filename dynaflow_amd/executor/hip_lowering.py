@@ -6,6 +6,7 @@ it deep-copies the sub-``GraphModule`` and replaces
 
 * ``linear(x, w)`` (no bias, bf16 or fp32)            -> ``dynaflow_hip.linear``
 * ``mul(silu(g), u)`` / ``mul(u, silu(g))``           -> ``dynaflow_hip.silu_mul``
+* ``rms_norm(x, (H,), w, eps)`` (bf16, last dim)      -> ``dynaflow_hip.rms_norm``
 
 With ``fuse_silu_epilogue`` a third rewrite follows: a ``silu_mul`` whose gate and up
 inputs are two bf16 ``linear`` nodes of the same activation becomes one
@@ -86,6 +87,29 @@ def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False) -> tuple[
     lowered = copy.deepcopy(gm)
     graph = lowered.graph
     stats = {"linear": 0, "silu_mul": 0}
+    if any(_target_name(n) == "rms_norm" and n.target is not ops.rms_norm for n in graph.nodes):
+        stats["rms_norm"] = 0
+        for node in list(graph.nodes):
+            if _target_name(node) != "rms_norm" or node.target is ops.rms_norm:
+                continue
+            args = list(node.args) + [None] * (4 - len(node.args))
+            x, shape = args[0], args[1]
+            weight = args[2] if args[2] is not None else node.kwargs.get("weight")
+            eps = args[3] if args[3] is not None else node.kwargs.get("eps")
+            ex, ew = _example(x), _example(weight)
+            if not isinstance(ex, torch.Tensor) or not isinstance(ew, torch.Tensor) or eps is None:
+                continue
+            h = _static_int(ex.shape[-1])
+            if ex.dtype != torch.bfloat16 or ew.dtype != torch.bfloat16 or h is None or h % 8 or h > 16384:
+                continue
+            if len(tuple(shape)) != 1:
+                continue
+            with graph.inserting_before(node):
+                new = graph.call_function(ops.rms_norm, (x, weight, float(eps)))
+            new.meta = dict(node.meta)
+            node.replace_all_uses_with(new)
+            graph.erase_node(node)
+            stats["rms_norm"] += 1
     if fuse_silu_epilogue:
         stats["gate_up_silu"] = 0
 

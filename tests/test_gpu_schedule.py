@@ -324,3 +324,62 @@ def test_fused_silu_epilogue_schedule():
     unfused = build(1024, 1024, 2816, torch.bfloat16)
     y0, _ = run(unfused[0], unfused[1], unfused[2], 1024)
     assert rel_err(y.float(), y0.float()) < TOL["bf16"]
+
+
+def build_decoder(batch, seq_len, hidden, heads, kv_heads, head_dim, inter, vocab, **knobs):
+    from dynaflow_amd.backend import make_backend
+    from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
+    from dynaflow_amd.decoder import DecoderLayer
+    from dynaflow_amd.manager import DynaFlowManager
+
+    layer = DecoderLayer(vocab=vocab, hidden=hidden, heads=heads, kv_heads=kv_heads, head_dim=head_dim, inter=inter,
+                         seq_len=seq_len, dtype=torch.bfloat16)
+    layer.init_weights(seed=7)
+    ids = torch.randint(0, vocab, (batch * seq_len,), generator=torch.Generator().manual_seed(4))
+    gpu_layer = DecoderLayer(vocab=vocab, hidden=hidden, heads=heads, kv_heads=kv_heads, head_dim=head_dim,
+                             inter=inter, seq_len=seq_len, dtype=torch.bfloat16, device="cuda")
+    gpu_layer.load_state_dict(layer.state_dict())
+    extra = {"min_nano_split_tokens": 1, "dump_graph": False}
+    extra.update(knobs)
+    cfg = DynaFlowConfig("dynaflow_amd.schedulers:DecoderOverlapScheduler", 2, InductorConfig(enabled=True),
+                         CUDAGraphConfig(enabled=False, capture_sizes=[batch * seq_len]), extra)
+    manager = DynaFlowManager()
+    torch._dynamo.reset()
+    idg = ids.cuda()
+    torch._dynamo.mark_dynamic(idg, 0)
+    compiled = torch.compile(gpu_layer, backend=make_backend(manager, cfg), fullgraph=True)
+    with torch.no_grad():
+        manager.prepare(batch, [seq_len] * batch)
+        compiled(idg)
+    return manager, compiled, idg, layer, ids
+
+
+def test_decoder_layer_attention_beside_mlp_small():
+    """Decoder layer through the manager: attention sub-graph of nano-batch 1 beside the MLP sub-graph of
+    nano-batch 0, against the independent float64 oracle (bf16 tolerance)."""
+    from dynaflow_amd import ops
+    from oracle import decoder as ref
+
+    batch, S = 4, 128
+    manager, compiled, idg, layer, ids = build_decoder(batch, S, 512, 8, 2, 64, 1408, 1000)
+    names = [n.target for n in manager.graph_module.graph.nodes if n.op == "call_module"]
+    mlp_graph = manager.graph_module.__dict__[names[1]].callable_dynamic
+    targets = [n.target for n in mlp_graph.graph.nodes if n.op == "call_function"]
+    assert ops.rms_norm in targets and ops.silu_mul in targets and targets.count(ops.linear) == 3
+    attn_targets = [n.target for n in manager.graph_module.__dict__[names[0]].callable_dynamic.graph.nodes
+                    if n.op == "call_function"]
+    assert attn_targets.count(ops.linear) == 4 and ops.rms_norm in attn_targets
+    with torch.no_grad():
+        split = manager.prepare(batch, [S] * batch)
+        y = compiled(idg)
+    torch.cuda.synchronize()
+    assert split.batch_indices == [0, 2, 4] and split.split_indices == [0, 2 * S, 4 * S]
+    assert manager.engine.issue_trace == [(names[0], 0), (names[1], 0), (names[0], 1), (names[1], 1)]
+    want = ref.decoder_layer(ids, ref.params_of(layer), S, 8, 2, 64)
+    assert rel_err(y.float(), want) < TOL["bf16"]
+    # serialised issue gives the same bits
+    m2, c2, idg2, _, _ = build_decoder(batch, S, 512, 8, 2, 64, 1408, 1000, serialize=True)
+    with torch.no_grad():
+        m2.prepare(batch, [S] * batch)
+        y2 = c2(idg2)
+    assert torch.equal(y, y2)
