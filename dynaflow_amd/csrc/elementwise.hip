@@ -173,6 +173,43 @@ transpose_bf16_kernel(const uint16_t* __restrict__ in, int64_t ld_in, uint16_t* 
   }
 }
 
+// Rotary embedding, half-split pairs (x[i], x[i + d/2]) of every head, position = row % seq_len:
+//   out_lo = lo*cos - hi*sin,  out_hi = hi*cos + lo*sin   (fp32, one rounding)
+// One lane rotates 8 pairs: 16 bytes of the low half and the matching 16 bytes of the high half.
+__global__ void __launch_bounds__(EW_THREADS)
+rope_bf16_kernel(const uint16_t* __restrict__ x, int64_t ld_x, uint16_t* __restrict__ out, int64_t ld_out,
+                 const float* __restrict__ cos_t, const float* __restrict__ sin_t, uint32_t groups, int heads,
+                 int half, int seq_len) {
+  const uint32_t gi = blockIdx.x * EW_THREADS + threadIdx.x;
+  if (gi >= groups) return;
+  const uint32_t per_head = half / 8;                 // groups of 8 pairs per head
+  const uint32_t per_row = per_head * heads;
+  const uint32_t row = gi / per_row;
+  const uint32_t in_row = gi - row * per_row;
+  const uint32_t head = in_row / per_head;
+  const uint32_t pair0 = (in_row - head * per_head) * 8;
+  const uint32_t pos = row % (uint32_t)seq_len;
+  const int64_t lo_off = (int64_t)head * (2 * half) + pair0;
+  const u32x4 lo = *reinterpret_cast<const u32x4*>(x + (int64_t)row * ld_x + lo_off);
+  const u32x4 hi = *reinterpret_cast<const u32x4*>(x + (int64_t)row * ld_x + lo_off + half);
+  const f32x4 c0 = *reinterpret_cast<const f32x4*>(cos_t + (int64_t)pos * half + pair0);
+  const f32x4 c1 = *reinterpret_cast<const f32x4*>(cos_t + (int64_t)pos * half + pair0 + 4);
+  const f32x4 s0 = *reinterpret_cast<const f32x4*>(sin_t + (int64_t)pos * half + pair0);
+  const f32x4 s1 = *reinterpret_cast<const f32x4*>(sin_t + (int64_t)pos * half + pair0 + 4);
+  u32x4 olo, ohi;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float c_a = w < 2 ? c0[2 * w] : c1[2 * w - 4], c_b = w < 2 ? c0[2 * w + 1] : c1[2 * w - 3];
+    const float s_a = w < 2 ? s0[2 * w] : s1[2 * w - 4], s_b = w < 2 ? s0[2 * w + 1] : s1[2 * w - 3];
+    const float lo_a = bf16_bits_to_f32(lo[w] & 0xffffu), lo_b = __uint_as_float(lo[w] & 0xffff0000u);
+    const float hi_a = bf16_bits_to_f32(hi[w] & 0xffffu), hi_b = __uint_as_float(hi[w] & 0xffff0000u);
+    olo[w] = pack2_bf16(lo_a * c_a - hi_a * s_a, lo_b * c_b - hi_b * s_b);
+    ohi[w] = pack2_bf16(hi_a * c_a + lo_a * s_a, hi_b * c_b + lo_b * s_b);
+  }
+  *reinterpret_cast<u32x4*>(out + (int64_t)row * ld_out + lo_off) = olo;
+  *reinterpret_cast<u32x4*>(out + (int64_t)row * ld_out + lo_off + half) = ohi;
+}
+
 __global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t* dst, uint32_t value, int64_t count) {
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t)gridDim.x * 256)
     dst[i] = value;
@@ -256,5 +293,23 @@ extern "C" int dfhip_fill_u32(void* dst, uint32_t value, int64_t count, dfhip_st
   if (blocks > 1024) blocks = 1024;
   hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<uint32_t*>(dst), value, count);
+  return dfhip_check_launch();
+}
+
+extern "C" int dfhip_rope_bf16(const void* x, int64_t ld_x, void* out, int64_t ld_out, const float* cos_table,
+                               const float* sin_table, int T, int heads, int head_dim, int seq_len,
+                               dfhip_stream_t stream) {
+  if (!x || !out || !cos_table || !sin_table) return DFHIP_ERR_NULL_POINTER;
+  if (T < 1 || heads < 1 || head_dim < 16 || head_dim % 16 != 0 || seq_len < 1) return DFHIP_ERR_BAD_SHAPE;
+  if ((int64_t)T * heads * (head_dim / 16) >= (int64_t)1 << 31) return DFHIP_ERR_BAD_SHAPE;
+  if (ld_x < (int64_t)heads * head_dim || ld_out < (int64_t)heads * head_dim) return DFHIP_ERR_BAD_STRIDE;
+  if (ld_x % 8 || ld_out % 8 || !dfhip_aligned16(x) || !dfhip_aligned16(out) || !dfhip_aligned16(cos_table) ||
+      !dfhip_aligned16(sin_table))
+    return DFHIP_ERR_BAD_ALIGNMENT;
+  const int half = head_dim / 2;
+  const uint32_t groups = (uint32_t)T * heads * (half / 8);
+  hipLaunchKernelGGL(rope_bf16_kernel, dim3((groups + EW_THREADS - 1) / EW_THREADS), dim3(EW_THREADS), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(x), ld_x,
+                     static_cast<uint16_t*>(out), ld_out, cos_table, sin_table, groups, heads, half, seq_len);
   return dfhip_check_launch();
 }

@@ -31,10 +31,13 @@ def rope_tables(seq_len: int, head_dim: int, theta: float, dtype=torch.float32, 
     return torch.cos(angles).to(dtype), torch.sin(angles).to(dtype)
 
 
+@torch._dynamo.allow_in_graph
 def apply_rope(t: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
     """Rotate pairs (t[..., i], t[..., i + d/2]) - the half-split convention of Llama checkpoints.
 
     ``t`` is [B, S, heads, d]; cos / sin are [S, d/2].  Arithmetic in fp32, one rounding.
+    Dynamo keeps a call of this function as ONE graph node (it does not trace into it), which the
+    HIP lowering replaces with the fused ``dynaflow_hip.rope`` kernel.
     """
     d2 = t.shape[-1] // 2
     tf = t.float()

@@ -7,6 +7,7 @@ it deep-copies the sub-``GraphModule`` and replaces
 * ``linear(x, w)`` (no bias, bf16 or fp32)            -> ``dynaflow_hip.linear``
 * ``mul(silu(g), u)`` / ``mul(u, silu(g))``           -> ``dynaflow_hip.silu_mul``
 * ``rms_norm(x, (H,), w, eps)`` (bf16, last dim)      -> ``dynaflow_hip.rms_norm``
+* ``apply_rope(t, cos, sin)`` (bf16, one graph node)  -> ``dynaflow_hip.rope``
 
 With ``fuse_silu_epilogue`` a third rewrite follows: a ``silu_mul`` whose gate and up
 inputs are two bf16 ``linear`` nodes of the same activation becomes one
@@ -154,6 +155,22 @@ def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False) -> tuple[
             graph.erase_node(silu)
             stats["silu_mul"] += 1
             break
+
+    for node in list(graph.nodes):
+        if _target_name(node) != "apply_rope" or len(node.args) != 3:
+            continue
+        et = _example(node.args[0])
+        if not isinstance(et, torch.Tensor) or et.dtype != torch.bfloat16 or et.dim() != 4:
+            continue
+        d = _static_int(et.shape[-1])
+        if d is None or d % 16:
+            continue
+        with graph.inserting_before(node):
+            new = graph.call_function(ops.rope, tuple(node.args))
+        new.meta = dict(node.meta)
+        node.replace_all_uses_with(new)
+        graph.erase_node(node)
+        stats["rope"] = stats.get("rope", 0) + 1
 
     if fuse_silu_epilogue:
         for node in list(graph.nodes):

@@ -230,7 +230,6 @@ class DynaFlowManager:
             bool(self.config.knob("whole_graph", False))
             and split.use_cudagraph
             and not split.is_dryrun
-            and list(split.num_tokens_padded) == list(split.num_tokens)
             and get_device().is_gpu
         )
 
@@ -252,7 +251,8 @@ class DynaFlowManager:
         """
         assert self.config is not None
         assert not kwargs, "whole-schedule graphs take positional graph inputs only"
-        eager_split = replace(split, use_cudagraph=False)
+        # the whole schedule is captured at its exact size: capture-size padding does not apply
+        eager_split = replace(split, use_cudagraph=False, num_tokens_padded=list(split.num_tokens))
         key = (
             tuple(split.split_indices),
             tuple((tuple(a.shape), a.dtype) if isinstance(a, torch.Tensor) else a for a in args),

@@ -35,6 +35,7 @@ _lib.define("gate_up_silu(Tensor x, Tensor w_gate, Tensor w_up) -> Tensor")
 _lib.define("rms_norm(Tensor x, Tensor weight, float eps) -> Tensor")
 _lib.define("add_rms_norm(Tensor x, Tensor residual, Tensor weight, float eps) -> (Tensor, Tensor)")
 _lib.define("transpose_weight(Tensor w) -> Tensor")
+_lib.define("rope(Tensor t, Tensor cos, Tensor sin) -> Tensor")
 _lib.define("quant_fp8(Tensor x) -> (Tensor, Tensor)")
 _lib.define("silu_mul_quant_fp8(Tensor gate, Tensor up) -> (Tensor, Tensor)")
 _lib.define("linear_fp8(Tensor x_q, Tensor w_q, Tensor x_scale, Tensor w_scale) -> Tensor")
@@ -255,6 +256,31 @@ torch.library.register_fake(
 )
 
 
+# ------------------------------------------------------------------ rope
+def _rope_impl(t: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """t [B, S, heads, d] bf16 (contiguous), cos/sin [S, d/2] fp32 -> rotated tensor of the same shape."""
+    _require_device(t, cos, sin)
+    lib = _cabi.load()
+    if t.dtype != torch.bfloat16 or cos.dtype != torch.float32 or sin.dtype != torch.float32 or t.dim() != 4:
+        raise RuntimeError("rope: t [B,S,heads,d] bf16 and fp32 tables expected")
+    B, S, heads, d = t.shape
+    if cos.shape != (S, d // 2) or sin.shape != (S, d // 2):
+        raise RuntimeError("rope: table shape mismatch")
+    src = t.contiguous()
+    out = torch.empty_like(src)
+    if src.numel() > 0:
+        rc = lib.dfhip_rope_bf16(
+            src.data_ptr(), heads * d, out.data_ptr(), heads * d, cos.contiguous().data_ptr(),
+            sin.contiguous().data_ptr(), B * S, heads, d, S, _stream(),
+        )
+        _cabi.check("dfhip_rope_bf16", rc)
+    return out
+
+
+_lib.impl("rope", _rope_impl, "CUDA")
+torch.library.register_fake("dynaflow_hip::rope", lambda t, cos, sin: torch.empty_like(t), lib=_lib)
+
+
 # ------------------------------------------------------ weight re-layout
 def _transpose_weight_impl(w: torch.Tensor) -> torch.Tensor:
     """[K, N] (``x @ W`` convention) -> [N, K] (``linear`` convention), bf16."""
@@ -372,6 +398,7 @@ gate_up_silu = torch.ops.dynaflow_hip.gate_up_silu
 rms_norm = torch.ops.dynaflow_hip.rms_norm
 add_rms_norm = torch.ops.dynaflow_hip.add_rms_norm
 transpose_weight = torch.ops.dynaflow_hip.transpose_weight
+rope = torch.ops.dynaflow_hip.rope
 quant_fp8 = torch.ops.dynaflow_hip.quant_fp8
 silu_mul_quant_fp8 = torch.ops.dynaflow_hip.silu_mul_quant_fp8
 linear_fp8 = torch.ops.dynaflow_hip.linear_fp8

@@ -158,6 +158,16 @@ int dfhip_silu_mul_f32(const void* gate, int64_t ld_gate, const void* up, int64_
 int dfhip_rmsnorm_bf16(const void* x, const void* residual, const void* weight, void* out,
                        void* residual_out, int M, int H, float eps, dfhip_stream_t stream);
 
+/* Rotary position embedding of x[T, heads*head_dim] (bf16), Llama half-split
+ * convention: pairs (x[i], x[i + head_dim/2]) of every head are rotated by the
+ * angle of position (row % seq_len), cos/sin tables [seq_len, head_dim/2] fp32;
+ * fp32 arithmetic, one rounding.  This is model code of the host framework in
+ * the reference (it reaches DynaFlow as a chain of elementwise FX nodes); here
+ * one launch.  head_dim % 16 == 0. */
+int dfhip_rope_bf16(const void* x, int64_t ld_x, void* out, int64_t ld_out, const float* cos_table,
+                    const float* sin_table, int T, int heads, int head_dim, int seq_len,
+                    dfhip_stream_t stream);
+
 /* out[N,K] = in[K,N]^T for bf16 matrices: packs a weight kept as [in, out]
  * (x @ W convention) into the [out, in] layout the GEMMs read.  K, N % 8 == 0. */
 int dfhip_transpose_bf16(const void* in, int64_t ld_in, void* out, int64_t ld_out, int K, int N,

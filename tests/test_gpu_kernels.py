@@ -299,3 +299,17 @@ def test_gate_up_silu_fused_epilogue(ops, M, I, K):
     # and against the two-kernel path at the bf16 tolerance
     two = ops.silu_mul(ops.linear(x.cuda(), wg.cuda()), ops.linear(x.cuda(), wu.cuda()), True)
     assert rel_err(got.float(), two.float()) < TOL["bf16"]
+
+
+@pytest.mark.parametrize("B,S,heads,d", [(1, 5, 1, 16), (3, 17, 4, 64), (2, 128, 8, 128)])
+def test_rope_against_complex_rotation(ops, B, S, heads, d):
+    from dynaflow_amd.decoder import rope_tables
+    from oracle import decoder as ref_decoder
+
+    t = randn((B, S, heads, d), 51).bfloat16()
+    cos, sin = rope_tables(S, d, 500000.0)
+    got = ops.rope(t.cuda(), cos.cuda(), sin.cuda())
+    want = ref_decoder.rope(t, 500000.0)          # float64 complex multiplication
+    assert got.shape == t.shape
+    assert bool(((got.float().cpu() - want.float()).abs() <= 2 ** -7 * want.float().abs() + 1e-6).all())
+    assert torch.equal(got[:, 0].cpu(), t[:, 0])  # position 0 is the identity

@@ -369,6 +369,7 @@ def test_decoder_layer_attention_beside_mlp_small():
     attn_targets = [n.target for n in manager.graph_module.__dict__[names[0]].callable_dynamic.graph.nodes
                     if n.op == "call_function"]
     assert attn_targets.count(ops.linear) == 4 and ops.rms_norm in attn_targets
+    assert attn_targets.count(ops.rope) == 2
     with torch.no_grad():
         split = manager.prepare(batch, [S] * batch)
         y = compiled(idg)
@@ -383,3 +384,21 @@ def test_decoder_layer_attention_beside_mlp_small():
         m2.prepare(batch, [S] * batch)
         y2 = c2(idg2)
     assert torch.equal(y, y2)
+
+
+def test_decoder_layer_whole_schedule_graph_with_padded_capture_size():
+    """use_cudagraph=True pads the nano-batch sizes to the capture size; the whole-schedule graph
+    ignores that padding (it captures the real sizes) and every replay equals the eager run."""
+    batch, S = 3, 64      # 128 + 64 tokens, only capture size 192: both nano-batches are padded
+    manager, compiled, idg, layer, ids = build_decoder(batch, S, 256, 4, 2, 64, 704, 500, whole_graph=True)
+    with torch.no_grad():
+        manager.prepare(batch, [S] * batch, use_cudagraph=False)
+        eager = compiled(idg).clone()
+        for i in range(3):
+            split = manager.prepare(batch, [S] * batch, use_cudagraph=True)
+            y = compiled(idg)
+            torch.cuda.synchronize()
+            assert list(split.num_tokens_padded) != list(split.num_tokens)
+            assert y.shape == eager.shape and torch.equal(y, eager), f"replay {i}"
+            torch.randn(256, 256, device="cuda").sum().item()
+    assert len(manager._schedule_graphs) == 1

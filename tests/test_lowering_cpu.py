@@ -62,3 +62,24 @@ def test_lowered_graph_fails_loudly_on_the_host():
     w = torch.randn(128, 64).bfloat16()
     with pytest.raises((RuntimeError, NotImplementedError)):
         head(x, 16, w, w)
+
+
+def test_decoder_layer_rope_and_norms_are_lowered():
+    from dynaflow_amd.decoder import DecoderLayer
+
+    captured = {}
+
+    def backend(gm, example_inputs):
+        captured["gm"] = gm
+        return gm
+
+    torch._dynamo.reset()
+    layer = DecoderLayer(vocab=64, hidden=128, heads=4, kv_heads=2, head_dim=32, inter=256, seq_len=8)
+    layer.init_weights(0)
+    ids = torch.arange(16) % 64
+    torch.compile(layer, backend=backend, fullgraph=True)(ids)
+    names = [getattr(n.target, "__name__", "") for n in captured["gm"].graph.nodes if n.op == "call_function"]
+    assert names.count("apply_rope") == 2          # q and k, each ONE node: dynamo does not trace into it
+    lowered, stats = lower_to_hip(captured["gm"])
+    assert stats["rope"] == 2 and stats["rms_norm"] == 2 and stats["linear"] == 7
+    assert targets(lowered).count(ops.rope) == 2
