@@ -36,7 +36,7 @@ if ROOT not in sys.path:
 TOKENS, HIDDEN, INTER, SPLITS = 4096, 4096, 14336, 2
 BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E
-GATE_GEMM_TRAFFIC_BYTES = 493.6e6  # measured with hardware counters; the summary is under profiles/
+GATE_GEMM_TRAFFIC_BYTES = 433.3e6  # measured with hardware counters; the summary is under profiles/
 METRIC = "MLP-layer tokens/s + overlap speedup vs serial, 8B-shape bf16, 1 MI355X"
 
 
@@ -418,7 +418,7 @@ def main() -> int:
             "unit": "TFLOP/s",
             "frac": gemm_flops / (ms_gate * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
             # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy of
-            # known size (fetch 370.7 MB + write 122.9 MB); algorithmic: 134.2 MB read + 58.7 MB written
+            # known size (fetch 370.9 MB + write 62.4 MB); algorithmic: 134.2 MB read + 58.7 MB written
             "traffic": GATE_GEMM_TRAFFIC_BYTES,
             "traffic_unit": "bytes per launch",
         },

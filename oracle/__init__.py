@@ -30,4 +30,14 @@ see the tests named below):
                     closed form, and the independent C restatement mlp_ref.c
                     (tests/test_oracle_mlp.py).  PARITY UNPINNED against the
                     reference's own outputs: the reference ships none.
+    decoder         one Llama-shaped decoder layer (embedding, RMSNorm, QKV,
+                    RoPE, causal grouped-query attention, output projection,
+                    residuals, SwiGLU MLP) in float64, written independently
+                    of the product module: RoPE as a complex multiplication,
+                    attention as an explicit masked softmax per head.  Pinned
+                    by special cases (position 0 is the identity, rotation
+                    preserves norms, one-token attention returns v, causal
+                    prefix independence) and by torch's own attention routine
+                    on the CPU  (tests/test_decoder_cpu.py).  PARITY UNPINNED
+                    against reference outputs: the reference ships none.
 """
