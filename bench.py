@@ -101,7 +101,7 @@ def time_steps(torch, manager, compiled, x, steps, warmup, use_graph):
     return (t1 - t0) * 1e3 / steps, y
 
 
-def time_kernel(torch, fn, iters, warmup=5):
+def time_kernel(torch, fn, iters, warmup=20):
     """Average duration of one launch, from HIP events on the stream it is launched on."""
     for _ in range(warmup):
         fn()

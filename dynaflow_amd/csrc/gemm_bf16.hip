@@ -220,8 +220,9 @@ DFHIP_DEVICE void wait_loaded(f32x4& v) { asm volatile("s_waitcnt vmcnt(0)" : "+
 // FUSED = true : C[M,N] = silu(A W^T) * (A W2^T) with W = gate weight, W2 = up weight, N = the
 //   intermediate size.  A tile is 256 rows x 128 columns; its "W half" holds 128 gate rows and 128 up
 //   rows arranged so that every wave owns gate AND up accumulators of the same 128x64 block (MFMA
-//   blocks j = 0,1 are gate, j = 2,3 are up): the SiLU*mul happens in registers, in fp32, on the
-//   unrounded projections, and only the product is written.
+//   blocks j = 0,1 are gate, j = 2,3 are up): the SiLU*mul happens in registers with the roundings
+//   of the two-kernel path (bf16 projections, bf16 silu, bf16 product) so that the result has the
+//   same bits, and only the product is written.
 template <bool FUSED>
 __global__ void __launch_bounds__(RTHREADS)
 gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
@@ -430,8 +431,10 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
           float p[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const float gt = acc[i][j][4 * g + e];
-            p[e] = (gt / (1.0f + expf(-gt))) * acc[i][j + 2][4 * g + e];
+            // the roundings of the two-kernel path: bf16 projections, bf16 silu, bf16 product
+            const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][4 * g + e]));
+            const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j + 2][4 * g + e]));
+            p[e] = bf16_bits_to_f32(f32_to_bf16_bits(gt / (1.0f + expf(-gt)))) * ut;
           }
           u32x2 v;
           v[0] = pack2_bf16(p[0], p[1]);
@@ -502,6 +505,228 @@ int launch_ring(const void* A, int64_t lda, const void* W, const void* W2, int64
   return dfhip_check_launch();
 }
 
+
+// ------------------------------------------------------------------ ring kernel, 256 x 224 tile
+// Same LDS-DMA ring as above with a tile of 256 rows x 224 columns: 4 waves stacked along M, each
+// 64 x 224 = 2 x 7 MFMA blocks (224 accumulator registers).  Column counts that are multiples of
+// 7 * 2^k (Llama's 14336 = 64 * 224) then give a tile count that divides evenly over the 256 CUs
+// (512 tiles instead of 448 of 256 x 256: 2 full rounds instead of 1.75 rounded up to 2).
+// FUSED: the W half holds 112 gate rows then 112 up rows; the wave parks both projections as
+// bf16 and the read-back pass computes bf16(bf16(silu(g)) * u) - the roundings of the two-kernel
+// path - and stores the [256, 112] block of the product.
+constexpr int TBN = 224;
+constexpr int TROW = TBN * 2 + 16;   // padded row of the staging area (bytes)
+
+template <bool FUSED>
+__global__ void __launch_bounds__(RTHREADS)
+gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
+                         const uint16_t* __restrict__ W2, uint16_t* __restrict__ C,
+                         int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n) {
+  constexpr int OUT_N = FUSED ? TBN / 2 : TBN;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  const int tile = remap_xcd(blockIdx.x, tiles_m * tiles_n);
+  const int per_panel = GROUP_M * tiles_n;
+  const int first_m = (tile / per_panel) * GROUP_M;
+  const int rows_in_panel = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+  const int in_panel = tile % per_panel;
+  const int m0 = (first_m + in_panel % rows_in_panel) * RBM;
+  const int n0 = (in_panel / rows_in_panel) * OUT_N;
+  const int KT = K / BK;
+
+  // DMA sources.  A half: 32 instructions of 8 rows, 8 per wave.  W half: 28 instructions, 7 per wave.
+  const uint8_t* a_src[8];
+  const uint8_t* w_src[7];
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    const int row = (wave * 8 + t) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    int ar = m0 + row; ar = ar < M ? ar : M - 1;
+    a_src[t] = reinterpret_cast<const uint8_t*>(A + (int64_t)ar * lda + chunk * 8);
+  }
+#pragma unroll
+  for (int t = 0; t < 7; ++t) {
+    const int row = (wave * 7 + t) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    if (FUSED) {
+      const bool up = row >= OUT_N;
+      int wr = n0 + (up ? row - OUT_N : row); wr = wr < N ? wr : N - 1;
+      w_src[t] = reinterpret_cast<const uint8_t*>((up ? W2 : W) + (int64_t)wr * ldw + chunk * 8);
+    } else {
+      int wr = n0 + row; wr = wr < N ? wr : N - 1;
+      w_src[t] = reinterpret_cast<const uint8_t*>(W + (int64_t)wr * ldw + chunk * 8);
+    }
+  }
+  auto dma_a = [&](int t, int slab, int unit) {
+    const int s = slab < KT ? slab : KT - 1;
+    dma16(unit * UNIT + (wave * 8 + t) * 1024, a_src[t] + (int64_t)s * (BK * 2));
+  };
+  auto dma_w = [&](int t, int slab, int unit) {
+    const int s = slab < KT ? slab : KT - 1;
+    dma16(unit * UNIT + (wave * 7 + t) * 1024, w_src[t] + (int64_t)s * (BK * 2));
+  };
+
+  const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
+  int koff[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) koff[ks] = ((2 * ks + fhalf) ^ fswz) * 16;
+  const int a_lane = (wave * 64 + frow) * 128, w_lane = frow * 128;
+
+  f32x16 acc[2][7];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 7; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_a(t, 0, 0);
+#pragma unroll
+  for (int t = 0; t < 7; ++t) dma_w(t, 0, 1);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_a(t, 1, 2);
+#pragma unroll
+  for (int t = 0; t < 7; ++t) dma_w(t, 1, 3);
+  wait_vmcnt<15>();   // slab 0 has landed; slab 1 may still be in flight
+  workgroup_barrier();
+
+  bf16x8 fa[2][2], fw[2][7];
+  // fragments in the order the MFMAs need them: A block 0, W blocks 0..6, A block 1
+  auto read_frag = [&](int idx, int ks, int slot, int unit_a, int unit_w) {
+    if (idx == 0 || idx == 8) {
+      const int i = idx >> 3;
+      fa[slot][i] = *reinterpret_cast<const bf16x8*>(smem + unit_a * UNIT + a_lane + koff[ks] + i * 4096);
+    } else {
+      fw[slot][idx - 1] = *reinterpret_cast<const bf16x8*>(smem + unit_w * UNIT + w_lane + koff[ks] + (idx - 1) * 4096);
+    }
+  };
+  auto mfma = [&](int q, int slot) {
+    const int i = q / 7, j = q % 7;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
+  };
+
+  int ua = 0, uw = 1;   // units of the slab being multiplied
+  int ia = 4, iw = 0;   // units that A(kt+2) and W(kt+2) go to
+#pragma unroll
+  for (int idx = 0; idx < 9; ++idx) read_frag(idx, 0, 0, ua, uw);
+  for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+    for (int q = 0; q < 14; ++q) {
+      mfma(q, 0);
+      if (q < 9) read_frag(q, 1, 1, ua, uw); else dma_a(q - 9, kt + 2, ia);
+      DFHIP_PIN;
+    }
+#pragma unroll
+    for (int q = 0; q < 14; ++q) {
+      mfma(q, 1);
+      if (q < 9) read_frag(q, 2, 0, ua, uw); else if (q < 12) dma_a(q - 4, kt + 2, ia);
+      DFHIP_PIN;
+    }
+#pragma unroll
+    for (int q = 0; q < 14; ++q) {
+      mfma(q, 0);
+      if (q < 9) read_frag(q, 3, 1, ua, uw);
+      DFHIP_PIN;
+    }
+    // all LDS reads of slab kt issued; slab kt+1 must have landed, only A(kt+2) may be in flight
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    wait_vmcnt<8>();
+    workgroup_barrier();
+    int na = ua + 2; if (na >= NUNITS) na -= NUNITS;
+    int nw = uw + 2; if (nw >= NUNITS) nw -= NUNITS;
+#pragma unroll
+    for (int q = 0; q < 14; ++q) {
+      mfma(q, 1);
+      if (q < 7) {
+        dma_w(q, kt + 2, iw);
+      } else if (q < 12) {
+        read_frag(q - 7, 0, 0, na, nw);
+      } else if (q == 12) {
+        read_frag(5, 0, 0, na, nw);
+        read_frag(6, 0, 0, na, nw);
+      } else {
+        read_frag(7, 0, 0, na, nw);
+        read_frag(8, 0, 0, na, nw);
+      }
+      DFHIP_PIN;
+    }
+    ua = na; uw = nw;
+    ia += 2; if (ia >= NUNITS) ia -= NUNITS;
+    iw += 2; if (iw >= NUNITS) iw -= NUNITS;
+  }
+  wait_vmcnt<0>();
+  workgroup_barrier();
+
+  // park 64 rows x 224 columns per wave as bf16, then store whole row pieces
+  uint8_t* park = smem + wave * (64 * TROW);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 7; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 v;
+        v[0] = pack2_bf16(acc[i][j][4 * g + 0], acc[i][j][4 * g + 1]);
+        v[1] = pack2_bf16(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+        *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * TROW + (j * 32 + g * 8 + fhalf * 4) * 2) = v;
+      }
+  DFHIP_PIN;
+  const int m_base = m0 + wave * 64;
+  if (FUSED) {
+#pragma unroll 2
+    for (int p = 0; p < 14; ++p) {
+      const int id = p * 64 + lane;
+      const int row = id / 14, c = id - row * 14;
+      const u32x4 g = *reinterpret_cast<const u32x4*>(park + row * TROW + c * 16);
+      const u32x4 u = *reinterpret_cast<const u32x4*>(park + row * TROW + (14 + c) * 16);
+      u32x4 v;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float g0 = bf16_bits_to_f32(g[w] & 0xffffu), g1 = __uint_as_float(g[w] & 0xffff0000u);
+        const float u0 = bf16_bits_to_f32(u[w] & 0xffffu), u1 = __uint_as_float(u[w] & 0xffff0000u);
+        const float s0 = bf16_bits_to_f32(f32_to_bf16_bits(g0 / (1.0f + expf(-g0))));
+        const float s1 = bf16_bits_to_f32(f32_to_bf16_bits(g1 / (1.0f + expf(-g1))));
+        v[w] = pack2_bf16(s0 * u0, s1 * u1);
+      }
+      const int m = m_base + row, n = n0 + c * 8;
+      if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+    }
+    return;
+  }
+#pragma unroll 4
+  for (int p = 0; p < 28; ++p) {
+    const int id = p * 64 + lane;
+    const int row = id / 28, c = id - row * 28;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * TROW + c * 16);
+    const int m = m_base + row, n = n0 + c * 8;
+    if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+  }
+}
+
+template <bool FUSED>
+int launch_ring224(const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw, void* C, int64_t ldc,
+                   int M, int N, int K, hipStream_t stream) {
+  auto kernel = gemm_bf16_ring224_kernel<FUSED>;
+  static bool lds_opted_in = false;
+  if (!lds_opted_in) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            RING_LDS) != hipSuccess)
+      return DFHIP_ERR_LAUNCH;
+    lds_opted_in = true;
+  }
+  constexpr int OUT_N = FUSED ? TBN / 2 : TBN;
+  const int tiles_m = (M + RBM - 1) / RBM;
+  const int tiles_n = (N + OUT_N - 1) / OUT_N;
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(RTHREADS), RING_LDS, stream,
+                     static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W),
+                     static_cast<const uint16_t*>(W2), static_cast<uint16_t*>(C), M, N, K, lda, ldw, ldc, tiles_m,
+                     tiles_n);
+  return dfhip_check_launch();
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 int launch(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
            int K, hipStream_t stream) {
@@ -520,6 +745,14 @@ int launch(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int6
                      static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W),
                      static_cast<uint16_t*>(C), M, N, K, lda, ldw, ldc, tiles_m, tiles_n);
   return dfhip_check_launch();
+}
+
+// Fraction of the CU-rounds that do work when [M, N] is cut into 256 x tile_n tiles and the
+// tiles are dealt to 256 CUs in rounds, weighted by the columns of a tile that exist.
+double round_fill(int M, int N, int tile_n) {
+  const int64_t tiles = (int64_t)((M + RBM - 1) / RBM) * ((N + tile_n - 1) / tile_n);
+  const int64_t rounds = (tiles + 255) / 256;
+  return (double)M * N / ((double)rounds * 256 * RBM * tile_n);
 }
 
 int check_args(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
@@ -545,6 +778,7 @@ extern "C" int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void
     case 1: return launch<256, 256, 2, 4>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 2: return launch<128, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 3: return launch<256, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
+    case 5: return launch_ring224<false>(A, lda, W, nullptr, ldw, C, ldc, M, N, K, s);
     default: return DFHIP_ERR_BAD_ARGUMENT;
   }
 }
@@ -564,6 +798,8 @@ extern "C" int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* spli
     if (s > 8) s = 8;
     while (s > 1 && K / BK < 16 * s) --s;   // keep at least 16 slabs per part
     if (s > 1) *split_k = s;
+    // 256 x 224 tiles when they fill the rounds of 256 workgroups clearly better (N = 7 * 2^k)
+    if (s <= 1 && round_fill(M, N, TBN) > round_fill(M, N, RBN) + 0.05) *variant = 5;
   }
   return DFHIP_OK;
 }
@@ -602,6 +838,8 @@ extern "C" int dfhip_gemm_bf16_gate_up_silu(const void* A, int64_t lda, const vo
   if (!W_up) return DFHIP_ERR_NULL_POINTER;
   if (int rc = check_args(A, lda, W_gate, ldw, Out, ldo, M, I, K)) return rc;
   if (!dfhip_aligned16(W_up)) return DFHIP_ERR_BAD_ALIGNMENT;
+  if (round_fill(M, I, TBN / 2) > round_fill(M, I, 128) + 0.05)
+    return launch_ring224<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, static_cast<hipStream_t>(stream));
   return launch_ring<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, 1, nullptr,
                            static_cast<hipStream_t>(stream));
 }

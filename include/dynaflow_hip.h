@@ -79,6 +79,8 @@ int dfhip_gemm_bf16_nt(const void* A, int64_t lda, const void* W, int64_t ldw, v
 
 /* Same contraction with an explicit kernel variant, for tuning and tests.
  * variant: 0 = 256x256 tile, LDS-DMA ring (the fast path);
+ *          5 = 256x224 tile, LDS-DMA ring (chosen when N = 7 * 2^k makes 224-wide
+ *              tiles fill the rounds of 256 workgroups better, e.g. N = 14336);
  *          register-staged tiles: 1 = 256x256 / 8 waves, 2 = 128x128 / 4 waves,
  *          3 = 256x128 / 4 waves, 4 = 256x256 / 4 waves. */
 int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
@@ -108,11 +110,11 @@ int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void* W, int64_t
 /* Gate and up projection with the SiLU*mul as the GEMM's epilogue:
  *   Out[M,I] = bf16( silu(A W_gate^T) * (A W_up^T) )
  * - the FX nodes linear, linear, silu, mul of the MLP in one launch.  Both
- * weights [I,K] with the same leading dimension ldw.  The SiLU and the product
- * are taken in fp32 on the unrounded projections (two separate kernels round
- * gate and up to bf16 first), so results differ from dfhip_gemm_bf16_nt +
- * dfhip_silu_mul_bf16 in the last bf16 bits.  Same shape rules as
- * dfhip_gemm_bf16_nt with N = I. */
+ * weights [I,K] with the same leading dimension ldw.  The epilogue applies
+ * the roundings of the separate kernels (projections to bf16, silu to bf16,
+ * product to bf16), so the result has the same bits as dfhip_gemm_bf16_nt
+ * (K not split) twice + dfhip_silu_mul_bf16 with round_silu = 1.  Same shape
+ * rules as dfhip_gemm_bf16_nt with N = I. */
 int dfhip_gemm_bf16_gate_up_silu(const void* A, int64_t lda, const void* W_gate, const void* W_up,
                                  int64_t ldw, void* Out, int64_t ldo, int M, int I, int K,
                                  dfhip_stream_t stream);

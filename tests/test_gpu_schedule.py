@@ -309,7 +309,7 @@ def test_fp8_config_full_size_properties():
 
 def test_fused_silu_epilogue_schedule():
     """fuse_silu_epilogue: {gate, up, silu, mul} becomes one GEMM with the SiLU*mul as epilogue, the cut
-    moves in front of the down projection; results stay within the bf16 tolerance of the oracle."""
+    moves in front of the down projection; same bits as the unfused schedule."""
     from dynaflow_amd import ops
 
     manager, compiled, xg, (x, wg, wu, wd) = build(1024, 1024, 2816, torch.bfloat16, fuse_silu_epilogue=True)
@@ -323,7 +323,7 @@ def test_fused_silu_epilogue_schedule():
     assert rel_err(y.float(), want) < TOL["bf16"]
     unfused = build(1024, 1024, 2816, torch.bfloat16)
     y0, _ = run(unfused[0], unfused[1], unfused[2], 1024)
-    assert rel_err(y.float(), y0.float()) < TOL["bf16"]
+    assert torch.equal(y, y0)   # the epilogue rounds like the separate kernels
 
 
 def build_decoder(batch, seq_len, hidden, heads, kv_heads, head_dim, inter, vocab, **knobs):
