@@ -20,6 +20,7 @@ dynaflow/runtime/engine.py:381.
 """
 from __future__ import annotations
 
+import math
 import os
 
 import torch
@@ -36,6 +37,10 @@ _lib.define("rms_norm(Tensor x, Tensor weight, float eps) -> Tensor")
 _lib.define("add_rms_norm(Tensor x, Tensor residual, Tensor weight, float eps) -> (Tensor, Tensor)")
 _lib.define("transpose_weight(Tensor w) -> Tensor")
 _lib.define("rope(Tensor t, Tensor cos, Tensor sin) -> Tensor")
+_lib.define(
+    "decode_attention(Tensor qkv, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor slots, Tensor lengths, "
+    "Tensor cos, Tensor sin, int q_heads, int kv_heads) -> Tensor"
+)
 _lib.define("quant_fp8(Tensor x) -> (Tensor, Tensor)")
 _lib.define("silu_mul_quant_fp8(Tensor gate, Tensor up) -> (Tensor, Tensor)")
 _lib.define("linear_fp8(Tensor x_q, Tensor w_q, Tensor x_scale, Tensor w_scale) -> Tensor")
@@ -281,6 +286,60 @@ _lib.impl("rope", _rope_impl, "CUDA")
 torch.library.register_fake("dynaflow_hip::rope", lambda t, cos, sin: torch.empty_like(t), lib=_lib)
 
 
+# ------------------------------------------------------- decode attention
+def _decode_attention_impl(qkv, k_cache, v_cache, slots, lengths, cos, sin, q_heads: int, kv_heads: int):
+    """RoPE + cache append + attention of one new token per sequence (see ``dynaflow_amd.decode``).
+
+    qkv [T, (q_heads + 2 kv_heads) * 128] bf16; k_cache [slots, kv_heads, capacity, 128];
+    v_cache [slots, kv_heads, capacity / 8, 128, 8]; slots, lengths [T] int32; cos, sin [rows, 64] fp32.
+    """
+    _require_device(qkv, k_cache, v_cache, slots, lengths, cos, sin)
+    lib = _cabi.load()
+    d = 128
+    if qkv.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise RuntimeError("decode_attention: bf16 tensors expected")
+    if slots.dtype != torch.int32 or lengths.dtype != torch.int32 or cos.dtype != torch.float32 or sin.dtype != torch.float32:
+        raise RuntimeError("decode_attention: int32 slots / lengths and fp32 tables expected")
+    if k_cache.dim() != 4 or v_cache.dim() != 5 or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise RuntimeError("decode_attention: contiguous k_cache [S,H,C,128] and v_cache [S,H,C/8,128,8] expected")
+    num_slots, kvh, capacity, hd = k_cache.shape
+    if hd != d or kvh != kv_heads or tuple(v_cache.shape) != (num_slots, kvh, capacity // 8, d, 8):
+        raise RuntimeError("decode_attention: cache shapes do not match")
+    if qkv.dim() != 2 or qkv.shape[1] != (q_heads + 2 * kv_heads) * d or qkv.stride(1) != 1:
+        raise RuntimeError("decode_attention: qkv [T, (q_heads + 2 kv_heads) * 128] expected")
+    T = qkv.shape[0]
+    if slots.shape != (T,) or lengths.shape != (T,) or cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != d // 2:
+        raise RuntimeError("decode_attention: slots / lengths / table shapes do not match")
+    slots, lengths, cos, sin = slots.contiguous(), lengths.contiguous(), cos.contiguous(), sin.contiguous()
+    out = torch.empty((T, q_heads * d), dtype=qkv.dtype, device=qkv.device)
+    if T > 0:
+        q_rot = torch.empty((T, q_heads * d), dtype=qkv.dtype, device=qkv.device)
+        stream = _stream()
+        rc = lib.dfhip_rope_kv_append_bf16(
+            qkv.data_ptr(), qkv.stride(0), q_rot.data_ptr(), q_heads * d, k_cache.data_ptr(), v_cache.data_ptr(),
+            slots.data_ptr(), lengths.data_ptr(), cos.data_ptr(), sin.data_ptr(), T, q_heads, kv_heads, d,
+            num_slots, capacity, cos.shape[0], stream,
+        )
+        _cabi.check("dfhip_rope_kv_append_bf16", rc)
+        rc = lib.dfhip_decode_attention_bf16(
+            q_rot.data_ptr(), q_heads * d, k_cache.data_ptr(), v_cache.data_ptr(), slots.data_ptr(),
+            lengths.data_ptr(), out.data_ptr(), q_heads * d, T, q_heads, kv_heads, d, num_slots, capacity,
+            1.0 / math.sqrt(d), stream,
+        )
+        _cabi.check("dfhip_decode_attention_bf16", rc)
+    return out
+
+
+_lib.impl("decode_attention", _decode_attention_impl, "CUDA")
+torch.library.register_fake(
+    "dynaflow_hip::decode_attention",
+    lambda qkv, k_cache, v_cache, slots, lengths, cos, sin, q_heads, kv_heads: qkv.new_empty(
+        (qkv.shape[0], q_heads * 128)
+    ),
+    lib=_lib,
+)
+
+
 # ------------------------------------------------------ weight re-layout
 def _transpose_weight_impl(w: torch.Tensor) -> torch.Tensor:
     """[K, N] (``x @ W`` convention) -> [N, K] (``linear`` convention), bf16."""
@@ -399,6 +458,7 @@ rms_norm = torch.ops.dynaflow_hip.rms_norm
 add_rms_norm = torch.ops.dynaflow_hip.add_rms_norm
 transpose_weight = torch.ops.dynaflow_hip.transpose_weight
 rope = torch.ops.dynaflow_hip.rope
+decode_attention = torch.ops.dynaflow_hip.decode_attention
 quant_fp8 = torch.ops.dynaflow_hip.quant_fp8
 silu_mul_quant_fp8 = torch.ops.dynaflow_hip.silu_mul_quant_fp8
 linear_fp8 = torch.ops.dynaflow_hip.linear_fp8

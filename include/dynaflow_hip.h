@@ -170,6 +170,38 @@ int dfhip_rope_bf16(const void* x, int64_t ld_x, void* out, int64_t ld_out, cons
                     const float* sin_table, int T, int heads, int head_dim, int seq_len,
                     dfhip_stream_t stream);
 
+/* Decode step against a static KV cache (bf16, head_dim 128).  Cache layout, per
+ * sequence slot and kv head, `capacity` positions (capacity % 32 == 0):
+ *   k_cache [num_slots][kv_heads][capacity][128]
+ *   v_cache [num_slots][kv_heads][capacity/8][128][8]   (8 consecutive positions
+ *                                                       of one dim are contiguous)
+ * Token t (one new token of sequence slot slots[t]) sits at position
+ * lengths[t] - 1; lengths[t] is the number of positions it attends to, itself
+ * included.  In the reference this is the host framework's attention custom op
+ * with its paged cache (an FX node the schedulers treat as opaque:
+ * examples/ae/scheduler/vllm/nanoflow.py:89-95 tags `unified_attention.*`
+ * "attention", "no-cudagraph"); here
+ * two kernels.
+ *
+ * dfhip_rope_kv_append_bf16: qkv[T, (q_heads + 2 kv_heads) * 128] holds q, k, v
+ *   of the new tokens; q and k are rotated (half-split pairs, cos/sin tables
+ *   [table_rows, 64] fp32, row = position), q goes to q_out[T, q_heads * 128], k
+ *   and v are written into the caches.  Tokens with slot or position out of range
+ *   leave the caches untouched.
+ * dfhip_decode_attention_bf16: out[T, q_heads * 128] = softmax(q K^T * scale) V
+ *   over positions 0 .. lengths[t]-1 of the token's slot, query head h reads kv
+ *   head h / (q_heads / kv_heads); q_heads / kv_heads <= 16.  Every cached
+ *   element is read once: HBM-bound.  A token whose slot is out of range or
+ *   whose length is < 1 gets zeros. */
+int dfhip_rope_kv_append_bf16(const void* qkv, int64_t ld_qkv, void* q_out, int64_t ld_q, void* k_cache,
+                              void* v_cache, const int32_t* slots, const int32_t* lengths,
+                              const float* cos_table, const float* sin_table, int T, int q_heads, int kv_heads,
+                              int head_dim, int num_slots, int capacity, int table_rows, dfhip_stream_t stream);
+int dfhip_decode_attention_bf16(const void* q, int64_t ld_q, const void* k_cache, const void* v_cache,
+                                const int32_t* slots, const int32_t* lengths, void* out, int64_t ld_out, int T,
+                                int q_heads, int kv_heads, int head_dim, int num_slots, int capacity, float scale,
+                                dfhip_stream_t stream);
+
 /* out[N,K] = in[K,N]^T for bf16 matrices: packs a weight kept as [in, out]
  * (x @ W convention) into the [out, in] layout the GEMMs read.  K, N % 8 == 0. */
 int dfhip_transpose_bf16(const void* in, int64_t ld_in, void* out, int64_t ld_out, int K, int N,
