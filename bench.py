@@ -36,7 +36,9 @@ if ROOT not in sys.path:
 TOKENS, HIDDEN, INTER, SPLITS = 4096, 4096, 14336, 2
 BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E
-GATE_GEMM_TRAFFIC_BYTES = 433.3e6  # measured with hardware counters; the summary is under profiles/
+# HBM-side bytes per launch, measured with hardware counters; the summaries are under profiles/
+GATE_GEMM_TRAFFIC_BYTES = 429.2e6      # fetch 370.5 MB + write 58.7 MB
+GATE_UP_SILU_TRAFFIC_BYTES = 797.8e6   # fetch 739.1 MB + write 58.7 MB
 METRIC = "MLP-layer tokens/s + overlap speedup vs serial, 8B-shape bf16, 1 MI355X"
 
 
@@ -52,6 +54,10 @@ def parse_args():
     p.add_argument("--fp8", action="store_true",
                    help="measure the fp8 70B-shaped MLP layer (x[8192,8192], I=28672, 4 nano-batches of 2048) "
                         "instead of the headline bf16 configuration")
+    p.add_argument("--decode-kernels", action="store_true",
+                   help="time the decode-step kernels at the shape of one nano-batch of the decode configuration "
+                        "(128 sequences, 32 query / 8 kv heads, 2048 cached positions): RoPE + cache append + "
+                        "attention, against the HBM roofline")
     p.add_argument("--decoder", action="store_true",
                    help="measure the full Llama-3-8B-shaped decoder layer (prefill 8 x 2048, attention of one "
                         "nano-batch beside the MLP of the other) instead of the headline configuration")
@@ -126,6 +132,7 @@ def single_kernels(torch, ops, x, weights, iters, calibration_copy=False):
         "gate_ms": time_kernel(torch, lambda: ops.linear(xb, weights[0]), iters),
         "down_ms": time_kernel(torch, lambda: ops.linear(act, weights[2]), iters),
         "silu_ms": time_kernel(torch, lambda: ops.silu_mul(gate, up, True), iters),
+        "gate_up_silu_ms": time_kernel(torch, lambda: ops.gate_up_silu(xb, weights[0], weights[1]), iters),
         "blas_ms": time_kernel(torch, lambda: torch.nn.functional.linear(xb, weights[0]), iters),
     }
     if calibration_copy:
@@ -133,6 +140,32 @@ def single_kernels(torch, ops, x, weights, iters, calibration_copy=False):
         dst = torch.empty_like(src)
         out["copy_256MiB_ms"] = time_kernel(torch, lambda: dst.copy_(src), iters)
     return out
+
+
+def decode_kernels(torch, ops, iters):
+    """Decode attention of one nano-batch (128 new tokens, each over 2048 cached positions of its own
+    sequence): every cached K and V element is read once, so the algorithmic bytes are the cache size."""
+    from dynaflow_amd.decoder import rope_tables
+
+    seqs, heads, kv_heads, capacity, d = 128, 32, 8, 2048, 128
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    k_cache = torch.randn(seqs, kv_heads, capacity, d, generator=gen, device="cuda").bfloat16()
+    v_cache = torch.randn(seqs, kv_heads, capacity // 8, d, 8, generator=gen, device="cuda").bfloat16()
+    qkv = torch.randn(seqs, (heads + 2 * kv_heads) * d, generator=gen, device="cuda").bfloat16()
+    slots = torch.arange(seqs, dtype=torch.int32, device="cuda")
+    lengths = torch.full((seqs,), capacity, dtype=torch.int32, device="cuda")
+    cos, sin = (t.cuda() for t in rope_tables(capacity, d, 500000.0))
+    ms = time_kernel(torch, lambda: ops.decode_attention(qkv, k_cache, v_cache, slots, lengths, cos, sin, heads,
+                                                         kv_heads), iters)
+    cache_bytes = 2.0 * seqs * kv_heads * capacity * d * 2
+    return {
+        "workload": f"decode attention, {seqs} sequences x {capacity} cached positions, {heads} query / "
+                    f"{kv_heads} kv heads, head_dim {d}, bf16 (rope + append kernel and attention kernel)",
+        "ms": ms,
+        "roofline": {"kernel": "decode_attention_kernel", "bound": "hbm", "achieved": cache_bytes / (ms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": cache_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "algorithmic_bytes": cache_bytes},
+    }
 
 
 def fp8_config(torch, steps, warmup):
@@ -316,6 +349,9 @@ def main() -> int:
     if args.decoder:
         print(json.dumps(decoder_config(torch, max(5, args.steps // 5), max(3, args.warmup // 5))))
         return 0
+    if args.decode_kernels:
+        print(json.dumps(decode_kernels(torch, ops, max(20, args.steps))))
+        return 0
     if args.fp8:
         print(json.dumps(fp8_config(torch, max(5, args.steps // 5), max(3, args.warmup // 5))))
         return 0
@@ -355,6 +391,7 @@ def main() -> int:
     # ---- single kernels, HIP events on the launching stream
     k = single_kernels(torch, ops, x, weights, max(20, args.steps))
     ms_gate, ms_down, ms_silu, ms_blas = k["gate_ms"], k["down_ms"], k["silu_ms"], k["blas_ms"]
+    ms_gus = k["gate_up_silu_ms"]
     mb = TOKENS // SPLITS
     gemm_flops = 2.0 * mb * HIDDEN * INTER          # one projection of one nano-batch
     silu_bytes = 3.0 * mb * INTER * 2               # read gate + up, write out
@@ -408,21 +445,38 @@ def main() -> int:
             "down_gemm": {"ms": ms_down, "tflops": gemm_flops / (ms_down * 1e-3) / 1e12},
             "silu_mul": {"ms": ms_silu, "gbs": silu_bytes / (ms_silu * 1e-3) / 1e9,
                          "frac_of_hbm_peak": silu_bytes / (ms_silu * 1e-3) / 1e9 / HBM_PEAK_GBS},
+            "gate_up_silu_gemm": {"ms": ms_gus, "tflops": 2 * gemm_flops / (ms_gus * 1e-3) / 1e12},
             "rocblas_same_gemm_for_scale": {"ms": ms_blas, "tflops": gemm_flops / (ms_blas * 1e-3) / 1e12},
         },
-        "roofline": {
-            "kernel": "gemm_bf16_nt (gate/up projection of one nano-batch: [2048,4096] x [14336,4096]^T)",
+    }
+    # the dominant kernel of the issue mode that `value` comes from
+    if fused_wins:
+        result["roofline"] = {
+            "kernel": "gemm_bf16_ring224_kernel<true> (gate and up projection of one nano-batch with the SiLU*mul "
+                      "epilogue: [2048,4096] x 2 x [14336,4096]^T -> act[2048,14336])",
+            "bound": "mfma",
+            "achieved": 2 * gemm_flops / (ms_gus * 1e-3) / 1e12,
+            "peak": BF16_MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": 2 * gemm_flops / (ms_gus * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
+            # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy of
+            # known size; algorithmic: 16.8 + 2 x 117.4 MB read, 58.7 MB written
+            "traffic": GATE_UP_SILU_TRAFFIC_BYTES,
+            "traffic_unit": "bytes per launch",
+        }
+    else:
+        result["roofline"] = {
+            "kernel": "gemm_bf16_ring224_kernel<false> (gate or up projection of one nano-batch: "
+                      "[2048,4096] x [14336,4096]^T)",
             "bound": "mfma",
             "achieved": gemm_flops / (ms_gate * 1e-3) / 1e12,
             "peak": BF16_MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": gemm_flops / (ms_gate * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
-            # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy of
-            # known size (fetch 370.9 MB + write 62.4 MB); algorithmic: 134.2 MB read + 58.7 MB written
+            # algorithmic: 134.2 MB read + 58.7 MB written
             "traffic": GATE_GEMM_TRAFFIC_BYTES,
             "traffic_unit": "bytes per launch",
-        },
-    }
+        }
     if not args.skip_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)
     else:
