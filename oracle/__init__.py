@@ -40,4 +40,12 @@ see the tests named below):
                     prefix independence) and by torch's own attention routine
                     on the CPU  (tests/test_decoder_cpu.py).  PARITY UNPINNED
                     against reference outputs: the reference ships none.
+    decode          one decode step (one new token per sequence) over stacked
+                    layers with KV caches, float64, caches in the natural
+                    layout, loops over tokens and heads.  Pinned by special
+                    cases (a single position returns its value, constant V,
+                    a dominated head), by token-by-token decoding == the
+                    prefill oracle on the whole sequence, and by the product
+                    module on the CPU  (tests/test_decode_cpu.py).  PARITY
+                    UNPINNED against reference outputs: there are none.
 """
