@@ -22,8 +22,15 @@ def decoder_split_rules() -> list[MatchingRule]:
     return [MatchingRule(condition=Mod(MLPBlock))]
 
 
+def _starts_at_compute_node(nodes, start: int) -> bool:
+    # Inside a sub-graph the placeholder that brings in the previous MLP block's output carries that
+    # block's module stack; without this veto the attention sub-graph of the next layer would match
+    # the Mod condition on that placeholder and be tagged as well.
+    return nodes[start].op != "placeholder"
+
+
 def decoder_tag_rules() -> dict[MatchingRule, set[str]]:
-    return {MatchingRule(condition=Mod(MLPBlock)): {MLP_TAG}}
+    return {MatchingRule(condition=Mod(MLPBlock), hook=_starts_at_compute_node): {MLP_TAG}}
 
 
 class DecoderOverlapScheduler(StaggeredScheduler):

@@ -200,3 +200,8 @@ def test_decode_schedule_on_recording_device(host_device):
     assert trace[0] == (subs[0], 0) and trace[1] == (subs[1], 0) and trace[2] == (subs[0], 1)
     for b in (0, 1):
         assert [name for name, batch in trace if batch == b] == subs
+    # attention sub-graphs on the main stream, MLP sub-graphs on the side stream, in every layer
+    streams = {e[1]: e[2] for e in host_device.log if e[0] == "range"}
+    for i, name in enumerate(subs):
+        for b in (0, 1):
+            assert streams[f"op_{name}_{b}"] == ("side" if i % 2 else "main"), (name, b)
