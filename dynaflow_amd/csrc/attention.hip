@@ -1,0 +1,284 @@
+// Causal grouped-query attention for prefill (bf16, head_dim 128), flash-attention style: scores and
+// probabilities never leave the registers.
+//
+// One workgroup = 256 query rows of one (sequence, query head); 4 waves x 64 rows.  K and V are staged
+// in LDS in blocks of 64 positions by LDS-DMA (3 stages in flight).  Both products are computed
+// transposed so that no operand ever needs a transpose:
+//   S^T[pos, qrow] = K Q^T   A = K rows from LDS, B = Q fragments held in registers for the whole kernel
+//   O^T[dim, qrow] = V^T P^T A = V in the blocked layout (8 consecutive positions of one dim are 16
+//                            contiguous bytes), B = P^T = the score accumulators themselves
+// MFMA row m of a score tile is mapped to position pi(m) (the two middle groups of 4 rows of every 16
+// are swapped) - K rows sit in LDS in that order - so that accumulator registers 0..7 of lane
+// (qrow, half) are the probabilities of positions 8*half .. 8*half+7: exactly the lane's B fragment of
+// the first 16-position k-step of P V; registers 8..15 are the second.  Every accumulator of a lane
+// belongs to the lane's own query row, so the softmax statistics and the rescaling are lane-local.
+#include "dfhip_common.h"
+
+namespace {
+
+constexpr int AD = 128;          // head dim
+constexpr int QROWS = 256;       // query rows per workgroup
+constexpr int KVB = 64;          // positions per staged block
+constexpr int STAGES = 3;
+constexpr int K_BYTES = KVB * AD * 2;            // 16 KiB
+constexpr int STAGE_BYTES = 2 * K_BYTES;         // K block + V block
+constexpr int ATT_LDS = STAGES * STAGE_BYTES;    // 96 KiB
+constexpr int OROW = AD * 2 + 16;                // padded row of the output staging area (bytes)
+constexpr float RESCALE_THRESHOLD = 8.0f;        // in units of log2: stale maxima up to 2^8 are tolerated
+
+DFHIP_DEVICE int pi(int m) {   // MFMA row -> position inside a 32-position tile
+  const int g = (m >> 2) & 3;
+  const int g2 = ((g & 1) << 1) | (g >> 1);      // 0,1,2,3 -> 0,2,1,3
+  return (m & 16) | (g2 << 2) | (m & 3);
+}
+
+__global__ void __launch_bounds__(256)
+causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint16_t* __restrict__ k, int64_t ld_k,
+                        const uint16_t* __restrict__ v_blk, uint16_t* __restrict__ out, int64_t ld_o, int B, int S,
+                        int q_heads, int kv_heads, float scale_log2) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 31, half = lane >> 5;
+  const int group = q_heads / kv_heads;
+  const int nqb = (S + QROWS - 1) / QROWS;
+
+  // workgroup -> (sequence, kv head, head in group, query block).  All query heads of a (sequence, kv
+  // head) pair run on ONE XCD (its K and V stay in that XCD's L2); inside an XCD's range the heavy query
+  // blocks (late rows, many K/V blocks) come first.
+  const int sets = B * kv_heads;
+  int b, kvh, hg, qb;
+  if (sets % 8 == 0) {
+    const int total = sets * group * nqb;
+    const int t = remap_xcd(blockIdx.x, total);
+    const int range = total / 8, sets_x = sets / 8;
+    const int local = t % range;
+    const int per_level = sets_x * group;
+    qb = nqb - 1 - local / per_level;
+    const int within = local % per_level;
+    const int set = (t / range) * sets_x + within / group;
+    hg = within % group;
+    b = set / kv_heads;
+    kvh = set % kv_heads;
+  } else {
+    const int t = blockIdx.x;
+    hg = t % group;
+    const int set = (t / group) % sets;
+    qb = nqb - 1 - t / (group * sets);
+    b = set / kv_heads;
+    kvh = set % kv_heads;
+  }
+  const int hq = kvh * group + hg;
+  const int q0 = qb * QROWS;                                  // first query row (inside the sequence)
+  const int last_block_wg = ((q0 + QROWS < S ? q0 + QROWS : S) + KVB - 1) / KVB - 1;
+  const int last_block_wave = q0 / KVB + wave;                 // the wave's diagonal block
+
+  // ---- DMA sources (per block: 4 K instructions + 4 V instructions per wave, 1 KiB each)
+  const uint16_t* kseq = k + (int64_t)b * S * ld_k + (int64_t)kvh * AD;
+  const uint8_t* vseq = reinterpret_cast<const uint8_t*>(v_blk) + ((int64_t)(b * kv_heads + kvh) * S) * (AD * 2);
+  int k_row_off[4];      // position offset inside the block for LDS row (wave*4 + t)*4 + lane/16
+  int k_chunk[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int row = (wave * 4 + t) * 4 + (lane >> 4);          // LDS row 0..63 (MFMA row order)
+    const int slot = lane & 15;
+    k_row_off[t] = (row & 32) | pi(row & 31);
+    k_chunk[t] = (slot & 8) | ((slot & 7) ^ (row & 7));        // logical 16-byte chunk held by this slot
+  }
+  auto issue_block = [&](int j, int stage) {
+    const int jj = j <= last_block_wg ? j : last_block_wg;     // past the end: re-read into a dead stage
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      int pos = jj * KVB + k_row_off[t];
+      pos = pos < S ? pos : S - 1;
+      dma16(stage * STAGE_BYTES + (wave * 4 + t) * 1024, kseq + (int64_t)pos * ld_k + k_chunk[t] * 8);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      dma16(stage * STAGE_BYTES + K_BYTES + (wave * 4 + t) * 1024,
+            vseq + (int64_t)jj * (KVB * AD * 2) + (wave * 4 + t) * 1024 + lane * 16);
+  };
+
+  // ---- Q fragments: B operand of S^T, lane supplies Q[qrow][16 ks + 8 half .. +8]
+  bf16x8 qf[2][8];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    int qrow = q0 + wave * 64 + nb * 32 + col;
+    qrow = qrow < S ? qrow : S - 1;
+    const uint16_t* qp = q + ((int64_t)b * S + qrow) * ld_q + (int64_t)hq * AD + 8 * half;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[nb][ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
+  }
+
+  f32x16 o[4][2];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[db][nb][r] = 0.0f;
+  float m_run[2] = {-INFINITY, -INFINITY};   // running (possibly stale) maximum of the raw scores
+  float l_run[2] = {0.0f, 0.0f};             // this lane's share of the row sum
+
+  issue_block(0, 0);
+  issue_block(1, 1);
+  const int k_read = col * 256;              // LDS row of this lane inside a 32-row tile
+  const int my_qrow0 = q0 + wave * 64 + col; // + 32 nb
+
+  for (int j = 0; j <= last_block_wg; ++j) {
+    const int stage = j % STAGES;
+    wait_vmcnt<8>();                         // block j has landed (block j+1 may be in flight)
+    workgroup_barrier();                     // ... for every wave; and everybody is done with block j-1
+    issue_block(j + 2, (j + 2) % STAGES);
+    if (j > last_block_wave) continue;       // beyond this wave's diagonal: only the staging duty
+    const bool diagonal = j == last_block_wave;
+    const uint8_t* kst = smem + stage * STAGE_BYTES;
+    const uint8_t* vst = kst + K_BYTES;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      f32x16 s[2];
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[nb][r] = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const int chunk = 2 * ks + half;
+        const int slot = (chunk & 8) | ((chunk & 7) ^ (col & 7));
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kst + sb * 8192 + k_read + slot * 16);
+        s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[0][ks], s[0], 0, 0, 0);
+        s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[1][ks], s[1], 0, 0, 0);
+      }
+      // register r of this lane: position p_base + 16*(r/8) + (r%8), query row my_qrow0 + 32 nb
+      const int p_base = j * KVB + sb * 32 + 8 * half;
+      bf16x8 pf[2][2];
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        if (diagonal) {
+          const int qrow = my_qrow0 + 32 * nb;
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (p_base + 16 * (r >> 3) + (r & 7) > qrow) s[nb][r] = -INFINITY;
+        }
+        float tmax = s[nb][0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, s[nb][r]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        // keep a stale maximum while the scores stay within 2^RESCALE_THRESHOLD of it
+        if (__any((tmax - m_run[nb]) * scale_log2 > RESCALE_THRESHOLD)) {
+          const float m_new = fmaxf(m_run[nb], tmax);
+          const float alpha = __builtin_amdgcn_exp2f((m_run[nb] - m_new) * scale_log2);   // 0 on the first block
+          m_run[nb] = m_new;
+          l_run[nb] *= alpha;
+#pragma unroll
+          for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[db][nb][r] *= alpha;
+        }
+        const float mc = m_run[nb] * scale_log2;
+        float lsum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[nb][r], scale_log2, -mc));
+          lsum += p;
+          pf[nb][r >> 3][r & 7] = static_cast<bf16_t>(p);
+        }
+        l_run[nb] += lsum;
+      }
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vst + ((sb * 4 + t * 2 + half) * AD + db * 32 + col) * 16);
+          o[db][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[0][t], o[db][0], 0, 0, 0);
+          o[db][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[1][t], o[db][1], 0, 0, 0);
+        }
+    }
+  }
+  wait_vmcnt<0>();        // the dead re-reads of the last iterations
+  workgroup_barrier();    // every wave is done with the stages: they become the output staging area
+
+  uint8_t* park = smem + wave * (64 * OROW);
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    const float l_tot = l_run[nb] + __shfl_xor(l_run[nb], 32, 64);
+    const float inv = 1.0f / l_tot;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w;
+        w[0] = pack2_bf16(o[db][nb][4 * g + 0] * inv, o[db][nb][4 * g + 1] * inv);
+        w[1] = pack2_bf16(o[db][nb][4 * g + 2] * inv, o[db][nb][4 * g + 3] * inv);
+        *reinterpret_cast<u32x2*>(park + (nb * 32 + col) * OROW + (db * 32 + 8 * g + 4 * half) * 2) = w;
+      }
+  }
+  DFHIP_PIN;
+  const int64_t row0 = (int64_t)b * S + q0 + wave * 64;
+#pragma unroll 4
+  for (int p = 0; p < 16; ++p) {
+    const int id = p * 64 + lane;
+    const int row = id >> 4, c = id & 15;
+    const u32x4 w = *reinterpret_cast<const u32x4*>(park + row * OROW + c * 16);
+    if (q0 + wave * 64 + row < S)
+      *reinterpret_cast<u32x4*>(out + (row0 + row) * ld_o + (int64_t)hq * AD + c * 8) = w;
+  }
+}
+
+// v[T, ld_v] (head h at column h*128) -> v_blk[B][kv_heads][S/8][128][8]
+__global__ void __launch_bounds__(128)
+pack_v_kernel(const uint16_t* __restrict__ v, int64_t ld_v, uint16_t* __restrict__ v_blk, int S, int kv_heads) {
+  const int pbs = S / 8;
+  const int pb = blockIdx.x % pbs;
+  const int h = (blockIdx.x / pbs) % kv_heads;
+  const int b = blockIdx.x / (pbs * kv_heads);
+  const int d = threadIdx.x;
+  const uint16_t* src = v + ((int64_t)b * S + pb * 8) * ld_v + (int64_t)h * AD + d;
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = (uint32_t)src[(2 * i) * ld_v] | ((uint32_t)src[(2 * i + 1) * ld_v] << 16);
+  u32x4 o = {w[0], w[1], w[2], w[3]};
+  *reinterpret_cast<u32x4*>(v_blk + ((((int64_t)b * kv_heads + h) * pbs + pb) * AD + d) * 8) = o;
+}
+
+}  // namespace
+
+extern "C" int dfhip_pack_v_bf16(const void* v, int64_t ld_v, void* v_blk, int B, int S, int kv_heads, int head_dim,
+                                 dfhip_stream_t stream) {
+  if (!v || !v_blk) return DFHIP_ERR_NULL_POINTER;
+  if (B < 1 || S < 8 || S % 8 != 0 || kv_heads < 1 || head_dim != AD ||
+      (int64_t)B * kv_heads * (S / 8) >= (int64_t)1 << 31)
+    return DFHIP_ERR_BAD_SHAPE;
+  if (ld_v < (int64_t)kv_heads * AD) return DFHIP_ERR_BAD_STRIDE;
+  if (!dfhip_aligned16(v_blk)) return DFHIP_ERR_BAD_ALIGNMENT;
+  hipLaunchKernelGGL(pack_v_kernel, dim3(B * kv_heads * (S / 8)), dim3(128), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(v), ld_v, static_cast<uint16_t*>(v_blk), S, kv_heads);
+  return dfhip_check_launch();
+}
+
+extern "C" int dfhip_causal_attention_bf16(const void* q, int64_t ld_q, const void* k, int64_t ld_k,
+                                           const void* v_blk, void* out, int64_t ld_o, int B, int S, int q_heads,
+                                           int kv_heads, int head_dim, float scale, dfhip_stream_t stream) {
+  if (!q || !k || !v_blk || !out) return DFHIP_ERR_NULL_POINTER;
+  if (B < 1 || S < KVB || S % KVB != 0 || q_heads < 1 || kv_heads < 1 || q_heads % kv_heads != 0 || head_dim != AD)
+    return DFHIP_ERR_BAD_SHAPE;
+  const int64_t groups = (int64_t)B * q_heads * ((S + QROWS - 1) / QROWS);
+  if (groups >= (int64_t)1 << 31) return DFHIP_ERR_BAD_SHAPE;
+  if (ld_q < (int64_t)q_heads * AD || ld_k < (int64_t)kv_heads * AD || ld_o < (int64_t)q_heads * AD)
+    return DFHIP_ERR_BAD_STRIDE;
+  if (ld_q % 8 || ld_k % 8 || ld_o % 8 || !dfhip_aligned16(q) || !dfhip_aligned16(k) || !dfhip_aligned16(v_blk) ||
+      !dfhip_aligned16(out))
+    return DFHIP_ERR_BAD_ALIGNMENT;
+  static bool lds_opted_in = false;
+  if (!lds_opted_in) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(causal_attention_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, ATT_LDS) != hipSuccess)
+      return DFHIP_ERR_LAUNCH;
+    lds_opted_in = true;
+  }
+  hipLaunchKernelGGL(causal_attention_kernel, dim3((unsigned)groups), dim3(256), ATT_LDS,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(q), ld_q,
+                     static_cast<const uint16_t*>(k), ld_k, static_cast<const uint16_t*>(v_blk),
+                     static_cast<uint16_t*>(out), ld_o, B, S, q_heads, kv_heads, scale * 1.4426950408889634f);
+  return dfhip_check_launch();
+}

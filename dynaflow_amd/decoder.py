@@ -46,6 +46,19 @@ def apply_rope(t: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
     return torch.cat((lo * c - hi * s, hi * c + lo * s), dim=-1).to(t.dtype)
 
 
+@torch._dynamo.allow_in_graph
+def causal_gqa_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    """Causal grouped-query attention: q [B, S, Hq, d], k / v [B, S, Hkv, d] -> [B, S, Hq, d].
+
+    ONE graph node for dynamo (it does not trace into it); the HIP lowering replaces it with the
+    ``dynaflow_hip.causal_attention`` kernel, this body is the definition in plain tensor operations.
+    """
+    out = F.scaled_dot_product_attention(
+        q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True, enable_gqa=True
+    )
+    return out.transpose(1, 2)
+
+
 class AttentionBlock(nn.Module):
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, seq_len: int, theta: float,
                  eps: float, dtype, device=None) -> None:
@@ -68,10 +81,7 @@ class AttentionBlock(nn.Module):
         v = F.linear(h, self.wv).view(-1, self.seq_len, self.kv_heads, self.head_dim)
         q = apply_rope(q, self.cos, self.sin)
         k = apply_rope(k, self.cos, self.sin)
-        attn = F.scaled_dot_product_attention(
-            q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True, enable_gqa=True
-        )
-        attn = attn.transpose(1, 2).reshape(-1, self.heads * self.head_dim)
+        attn = causal_gqa_attention(q, k, v).reshape(-1, self.heads * self.head_dim)
         return x + F.linear(attn, self.wo)
 
 

@@ -9,6 +9,7 @@ it deep-copies the sub-``GraphModule`` and replaces
 * ``rms_norm(x, (H,), w, eps)`` (bf16, last dim)      -> ``dynaflow_hip.rms_norm``
 * ``apply_rope(t, cos, sin)`` (bf16, one graph node)  -> ``dynaflow_hip.rope``
 * ``attend_and_append(qkv, k_cache, v_cache, ...)``   -> ``dynaflow_hip.decode_attention``
+* ``causal_gqa_attention(q, k, v)`` (bf16, d 128, S%64) -> ``dynaflow_hip.causal_attention``
 
 With ``fuse_silu_epilogue`` a third rewrite follows: a ``silu_mul`` whose gate and up
 inputs are two bf16 ``linear`` nodes of the same activation becomes one
@@ -172,6 +173,22 @@ def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False) -> tuple[
         node.replace_all_uses_with(new)
         graph.erase_node(node)
         stats["rope"] = stats.get("rope", 0) + 1
+
+    for node in list(graph.nodes):
+        if _target_name(node) != "causal_gqa_attention" or len(node.args) != 3:
+            continue
+        et = _example(node.args[0])
+        if not isinstance(et, torch.Tensor) or et.dtype != torch.bfloat16 or et.dim() != 4:
+            continue
+        seq, d = _static_int(et.shape[1]), _static_int(et.shape[3])
+        if seq is None or seq % 64 or d != 128:
+            continue
+        with graph.inserting_before(node):
+            new = graph.call_function(ops.causal_attention, tuple(node.args))
+        new.meta = dict(node.meta)
+        node.replace_all_uses_with(new)
+        graph.erase_node(node)
+        stats["causal_attention"] = stats.get("causal_attention", 0) + 1
 
     for node in list(graph.nodes):
         if _target_name(node) != "attend_and_append" or len(node.args) != 9:

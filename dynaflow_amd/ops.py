@@ -37,6 +37,7 @@ _lib.define("rms_norm(Tensor x, Tensor weight, float eps) -> Tensor")
 _lib.define("add_rms_norm(Tensor x, Tensor residual, Tensor weight, float eps) -> (Tensor, Tensor)")
 _lib.define("transpose_weight(Tensor w) -> Tensor")
 _lib.define("rope(Tensor t, Tensor cos, Tensor sin) -> Tensor")
+_lib.define("causal_attention(Tensor q, Tensor k, Tensor v) -> Tensor")
 _lib.define(
     "decode_attention(Tensor qkv, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor slots, Tensor lengths, "
     "Tensor cos, Tensor sin, int q_heads, int kv_heads) -> Tensor"
@@ -286,6 +287,47 @@ _lib.impl("rope", _rope_impl, "CUDA")
 torch.library.register_fake("dynaflow_hip::rope", lambda t, cos, sin: torch.empty_like(t), lib=_lib)
 
 
+# ------------------------------------------------------ prefill attention
+def _token_rows(t: torch.Tensor, what: str):
+    """[B, S, H, 128] with contiguous heads -> (tensor, token stride in elements)."""
+    if t.dim() != 4 or t.shape[3] != 128 or t.stride(3) != 1 or t.stride(2) != 128 or t.stride(0) != t.shape[1] * t.stride(1):
+        t = t.contiguous()
+    return t, t.stride(1)
+
+
+def _causal_attention_impl(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    """q [B, S, Hq, 128], k / v [B, S, Hkv, 128] (bf16) -> softmax(q k^T / sqrt(128), causal) v as [B, S, Hq, 128]."""
+    _require_device(q, k, v)
+    lib = _cabi.load()
+    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
+        raise RuntimeError("causal_attention: bf16 tensors expected")
+    if q.dim() != 4 or k.dim() != 4 or v.shape != k.shape or q.shape[:2] != k.shape[:2] or q.shape[3] != 128 or k.shape[3] != 128:
+        raise RuntimeError("causal_attention: q [B,S,Hq,128] and k, v [B,S,Hkv,128] expected")
+    B, S, Hq, d = q.shape
+    Hkv = k.shape[2]
+    if S % 64 != 0 or Hq % Hkv != 0:
+        raise RuntimeError("causal_attention: sequence length must be a multiple of 64, q heads a multiple of kv heads")
+    q, ld_q = _token_rows(q, "q")
+    k, ld_k = _token_rows(k, "k")
+    v, ld_v = _token_rows(v, "v")
+    out = torch.empty((B, S, Hq, d), dtype=q.dtype, device=q.device)
+    if B > 0:
+        v_blk = torch.empty((B, Hkv, S // 8, d, 8), dtype=q.dtype, device=q.device)
+        stream = _stream()
+        rc = lib.dfhip_pack_v_bf16(v.data_ptr(), ld_v, v_blk.data_ptr(), B, S, Hkv, d, stream)
+        _cabi.check("dfhip_pack_v_bf16", rc)
+        rc = lib.dfhip_causal_attention_bf16(
+            q.data_ptr(), ld_q, k.data_ptr(), ld_k, v_blk.data_ptr(), out.data_ptr(), Hq * d, B, S, Hq, Hkv, d,
+            1.0 / math.sqrt(d), stream,
+        )
+        _cabi.check("dfhip_causal_attention_bf16", rc)
+    return out
+
+
+_lib.impl("causal_attention", _causal_attention_impl, "CUDA")
+torch.library.register_fake("dynaflow_hip::causal_attention", lambda q, k, v: torch.empty_like(q), lib=_lib)
+
+
 # ------------------------------------------------------- decode attention
 def _decode_attention_impl(qkv, k_cache, v_cache, slots, lengths, cos, sin, q_heads: int, kv_heads: int):
     """RoPE + cache append + attention of one new token per sequence (see ``dynaflow_amd.decode``).
@@ -459,6 +501,7 @@ add_rms_norm = torch.ops.dynaflow_hip.add_rms_norm
 transpose_weight = torch.ops.dynaflow_hip.transpose_weight
 rope = torch.ops.dynaflow_hip.rope
 decode_attention = torch.ops.dynaflow_hip.decode_attention
+causal_attention = torch.ops.dynaflow_hip.causal_attention
 quant_fp8 = torch.ops.dynaflow_hip.quant_fp8
 silu_mul_quant_fp8 = torch.ops.dynaflow_hip.silu_mul_quant_fp8
 linear_fp8 = torch.ops.dynaflow_hip.linear_fp8
