@@ -284,7 +284,8 @@ def decoder_config(torch, steps, warmup):
         "data": "synthetic",
         "config": {"workload": "Llama-3-8B-shaped decoder layer, prefill 8 x 2048 tokens, 2 nano-batches of 4 "
                                "sequences, attention sub-graph of one beside the MLP sub-graph of the other; "
-                               "attention itself on PyTorch's fused kernel, projections/MLP/norms on HIP operators"},
+                               "projections, RoPE, causal attention, norms and MLP on the hand-written HIP "
+                               "operators (embedding gather, residual adds and the final concatenation on aten)"},
         "timings": results,
         "layer": {"algorithmic_tflop": flops / 1e12, "tflops": flops / (best * 1e-3) / 1e12,
                   "frac_of_bf16_mfma_peak": flops / (best * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS},

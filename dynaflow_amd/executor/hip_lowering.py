@@ -52,6 +52,19 @@ def _static_int(value: Any) -> int | None:
     return value if isinstance(value, int) and not isinstance(value, torch.SymInt) else None
 
 
+def _traced_int(value: Any) -> int | None:
+    """A dimension as a number: a plain int, or the value a symbolic dimension had while tracing.
+
+    ``view(-1, seq_len, ...)`` of a token-shaped tensor leaves dynamo with an unsimplified
+    expression such as ``s // (s // seq_len)`` for the constant ``seq_len``.  The operator that is
+    put in checks the real size again at run time and raises if it cannot handle it.
+    """
+    if isinstance(value, torch.SymInt):
+        hint = getattr(value.node, "hint", None)
+        return int(hint) if hint is not None else None
+    return value if isinstance(value, int) else None
+
+
 def _linear_supported(x: Any, w: Any) -> bool:
     ex, ew = _example(x), _example(w)
     if not isinstance(ex, torch.Tensor) or not isinstance(ew, torch.Tensor):
@@ -180,7 +193,7 @@ def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False) -> tuple[
         et = _example(node.args[0])
         if not isinstance(et, torch.Tensor) or et.dtype != torch.bfloat16 or et.dim() != 4:
             continue
-        seq, d = _static_int(et.shape[1]), _static_int(et.shape[3])
+        seq, d = _traced_int(et.shape[1]), _static_int(et.shape[3])
         if seq is None or seq % 64 or d != 128:
             continue
         with graph.inserting_before(node):

@@ -83,3 +83,34 @@ def test_decoder_layer_rope_and_norms_are_lowered():
     lowered, stats = lower_to_hip(captured["gm"])
     assert stats["rope"] == 2 and stats["rms_norm"] == 2 and stats["linear"] == 7
     assert targets(lowered).count(ops.rope) == 2
+
+
+def test_decoder_layer_attention_is_lowered_for_head_dim_128():
+    from dynaflow_amd.decoder import DecoderLayer
+
+    captured = {}
+
+    def backend(gm, example_inputs):
+        captured["gm"] = gm
+        return gm
+
+    torch._dynamo.reset()
+    layer = DecoderLayer(vocab=64, hidden=256, heads=4, kv_heads=2, head_dim=128, inter=256, seq_len=64)
+    layer.init_weights(0)
+    ids = torch.arange(128) % 64
+    torch._dynamo.mark_dynamic(ids, 0)
+    torch.compile(layer, backend=backend, fullgraph=True)(ids)
+    names = [getattr(n.target, "__name__", "") for n in captured["gm"].graph.nodes if n.op == "call_function"]
+    assert names.count("causal_gqa_attention") == 1            # one node: dynamo does not trace into it
+    lowered, stats = lower_to_hip(captured["gm"])
+    assert stats["causal_attention"] == 1 and stats["rope"] == 2
+    assert targets(lowered).count(ops.causal_attention) == 1
+    # a sequence length the kernel does not take (not a multiple of 64) stays on the tensor operations
+    torch._dynamo.reset()
+    layer = DecoderLayer(vocab=64, hidden=256, heads=4, kv_heads=2, head_dim=128, inter=256, seq_len=48)
+    layer.init_weights(0)
+    ids = torch.arange(96) % 64
+    torch._dynamo.mark_dynamic(ids, 0)
+    torch.compile(layer, backend=backend, fullgraph=True)(ids)
+    _, stats = lower_to_hip(captured["gm"])
+    assert "causal_attention" not in stats
