@@ -88,3 +88,17 @@ def test_causal_attention_full_size_properties(ops):
     fused = torch.nn.functional.scaled_dot_product_attention(
         q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True, enable_gqa=True).transpose(1, 2)
     assert rel_err(got.float(), fused.float()) < TOL_BF16
+
+
+def test_causal_attention_under_graph_capture(ops):
+    q, k, v = (t.cuda() for t in inputs(2, 256, 4, 2, 21))
+    eager = ops.causal_attention(q, k, v).clone()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = ops.causal_attention(q, k, v)
+    for i in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {i}"
+        torch.randn(256, 256, device="cuda").sum().item()

@@ -192,3 +192,38 @@ def test_decode_schedule_against_oracle_and_graph_replay():
     for i, blk in enumerate(model.attn):
         got_k = blk.k_cache.double().cpu().permute(0, 2, 1, 3)
         assert (got_k - kc[i]).abs().max() <= 0.05 * kc[i].abs().max()
+
+
+def test_decode_attention_under_graph_capture(ops):
+    """The entry points allocate nothing and synchronise nothing, so the operator can be captured into a
+    hipGraph: every replay (with eager work between replays) must equal the eager result, and a replay picks
+    up new contents of the captured tensors."""
+    from dynaflow_amd.decode import pack_v_cache
+    from dynaflow_amd.decoder import rope_tables
+
+    T, heads, kv_heads, capacity = 12, 8, 2, 128
+    g = torch.Generator().manual_seed(2)
+    k_cache = torch.randn(T + 3, kv_heads, capacity, D, generator=g).bfloat16().cuda()
+    v_cache = pack_v_cache(torch.randn(T + 3, kv_heads, capacity, D, generator=g).bfloat16()).cuda()
+    qkv = torch.randn(T, (heads + 2 * kv_heads) * D, generator=g).bfloat16().cuda()
+    slots = torch.randperm(T + 3, generator=g)[:T].int().cuda()
+    lens = torch.randint(1, capacity + 1, (T,), generator=g).int().cuda()
+    cos, sin = (t.cuda() for t in rope_tables(capacity, D, 500000.0))
+    print("decode attention: eager", flush=True)
+    eager = ops.decode_attention(qkv, k_cache, v_cache, slots, lens, cos, sin, heads, kv_heads).clone()
+    torch.cuda.synchronize()
+    print("decode attention: capture", flush=True)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = ops.decode_attention(qkv, k_cache, v_cache, slots, lens, cos, sin, heads, kv_heads)
+    for i in range(3):
+        print(f"decode attention: replay {i}", flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {i}"
+        torch.randn(256, 256, device="cuda").sum().item()
+    qkv.copy_(torch.randn(qkv.shape, generator=g).bfloat16())
+    graph.replay()
+    torch.cuda.synchronize()
+    want = ops.decode_attention(qkv, k_cache, v_cache, slots, lens, cos, sin, heads, kv_heads)
+    assert torch.equal(out, want) and not torch.equal(out, eager)
