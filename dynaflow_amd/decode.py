@@ -9,9 +9,10 @@ these pieces).  This module is that graph for the build's own measurements:
   two-stream schedule can be captured once and replayed;
 * every token carries its cache slot and its attention length (``slots``, ``lengths``: token-shaped
   inputs, cut per nano-batch by the engine like the activations);
-* ``attend_and_append`` is ONE graph node (dynamo does not trace into it); on the GPU the HIP
-  lowering replaces it with ``dynaflow_hip.decode_attention``; its body below is the definition in
-  plain tensor operations, used on the host.
+* ``attend_and_append`` is an operator of its own (``dynaflow_model::attend_and_append``, declared
+  to mutate the two caches), so it is ONE graph node; on the GPU the HIP lowering replaces it with
+  ``dynaflow_hip.decode_attention``; its body below is the definition in plain tensor operations,
+  used on the host.
 
 Cache layout (head_dim 128): ``k_cache [slots, kv_heads, capacity, 128]``,
 ``v_cache [slots, kv_heads, capacity / 8, 128, 8]`` (8 consecutive positions of one dim contiguous).
@@ -41,7 +42,7 @@ def unpack_v_cache(v_cache: torch.Tensor) -> torch.Tensor:
     return v_cache.permute(0, 1, 2, 4, 3).reshape(s, h, blocks * 8, d)
 
 
-@torch._dynamo.allow_in_graph
+@torch.library.custom_op("dynaflow_model::attend_and_append", mutates_args=("k_cache", "v_cache"))
 def attend_and_append(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slots: torch.Tensor,
                       lengths: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, q_heads: int,
                       kv_heads: int) -> torch.Tensor:
@@ -49,6 +50,9 @@ def attend_and_append(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
 
     Token t belongs to cache slot ``slots[t]``, sits at position ``lengths[t] - 1`` and attends to
     positions ``0 .. lengths[t] - 1``.  qkv is ``[T, (q_heads + 2 kv_heads) * 128]``.
+
+    Declared as an operator that mutates the two caches: a function that writes to its inputs must not
+    be handed to dynamo as a plain in-graph function.
     """
     T, d = qkv.shape[0], HEAD_DIM
     capacity = k_cache.shape[2]
@@ -73,6 +77,11 @@ def attend_and_append(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
     scores = scores.masked_fill(masked[:, None, None, :], float("-inf"))
     out = torch.einsum("tkgp,tkpd->tkgd", torch.softmax(scores, dim=-1), values)
     return out.reshape(T, q_heads * d).to(qkv.dtype)
+
+
+@attend_and_append.register_fake
+def _(qkv, k_cache, v_cache, slots, lengths, cos, sin, q_heads, kv_heads):
+    return qkv.new_empty((qkv.shape[0], q_heads * HEAD_DIM))
 
 
 class DecodeAttentionBlock(nn.Module):

@@ -39,7 +39,10 @@ _MUL_TARGETS = {operator.mul, torch.mul}
 def _target_name(node: fx.Node) -> str | None:
     if node.op != "call_function":
         return None
-    return getattr(node.target, "__name__", None)
+    name = getattr(node.target, "__name__", None)
+    if isinstance(node.target, torch._ops.OpOverload):   # "name.overload" -> "name"
+        name = node.target.overloadpacket.__name__
+    return name
 
 
 def _example(node: Any) -> Any:

@@ -91,6 +91,9 @@ class _ScheduleGraph:
         self.output = output
 
 
+MAX_WHOLE_GRAPH_SEGMENTS = 2
+
+
 class DynaFlowManager:
     """Splits a traced graph and runs it under a programmable scheduler."""
 
@@ -251,6 +254,17 @@ class DynaFlowManager:
         """
         assert self.config is not None
         assert not kwargs, "whole-schedule graphs take positional graph inputs only"
+        assert self.graph_module is not None
+        segments = sum(1 for n in self.graph_module.graph.nodes if n.op == "call_module")
+        if segments > MAX_WHOLE_GRAPH_SEGMENTS:
+            # Ending the stream capture of a six-segment, two-stream schedule crashed inside the runtime
+            # (segmentation fault in the capture's end call); two segments per nano-batch, with up to
+            # four nano-batches, capture and replay correctly.  Until the cause is known the larger
+            # schedules are not captured as one graph: use per-sub-graph graphs or the eager schedule.
+            raise NotImplementedError(
+                f"whole-schedule capture is limited to {MAX_WHOLE_GRAPH_SEGMENTS} sub-graphs per nano-batch "
+                f"(this graph has {segments})"
+            )
         # the whole schedule is captured at its exact size: capture-size padding does not apply
         eager_split = replace(split, use_cudagraph=False, num_tokens_padded=list(split.num_tokens))
         key = (

@@ -154,18 +154,15 @@ def build_decode(T, whole_graph, **over):
     return manager, compiled, dev, host, model, (ids, slots, lengths), cfg_model
 
 
-@pytest.mark.skip(reason="the test process aborted (fatal signal, no GPU fault reported) on its first run on the GPU and "
-                         "the cause has not been found on the host: the host flow passes with stand-in operators, the "
-                         "kernels' address arithmetic is in bounds for this configuration, the kernel tests above pass; "
-                         "stays off the GPU until a cause is shown")
-def test_decode_schedule_against_oracle_and_graph_replay():
-    """Three layers, 24 sequences, two nano-batches: every sub-graph runs on HIP operators, the result matches
-    the float64 oracle, and the whole-schedule graph replays to the same bits (a decode step with fixed
-    lengths rewrites the same cache entries, so replays are idempotent)."""
+def test_decode_schedule_against_oracle():
+    """Three layers, 24 sequences, two nano-batches on two streams: every sub-graph runs on HIP operators
+    (attention sub-graphs on the main stream, MLP sub-graphs on the side stream) and the result matches the
+    float64 oracle, as do the appended cache entries."""
     from dynaflow_amd import ops
 
     T = 24
-    manager, compiled, dev, host, model, (ids, slots, lengths), cm = build_decode(T, whole_graph=True)
+    print("decode schedule: build (trace, lower, first call on the fast path)", flush=True)
+    manager, compiled, dev, host, model, (ids, slots, lengths), cm = build_decode(T, whole_graph=False)
     subs = [n.target for n in manager.graph_module.graph.nodes if n.op == "call_module"]
     assert len(subs) == 6
     attn_targets = [n.target for n in manager.graph_module.__dict__[subs[0]].callable_dynamic.graph.nodes
@@ -175,23 +172,38 @@ def test_decode_schedule_against_oracle_and_graph_replay():
     kc, vc = ref.caches_of(host)
     want = ref.decode_step(ids, slots, lengths, params, kc, vc, cm["heads"], cm["kv_heads"])
     with torch.no_grad():
+        print("decode schedule: eager two-stream run", flush=True)
         split = manager.prepare(T, [1] * T, use_cudagraph=False)
-        eager = compiled(*dev).clone()
+        y = compiled(*dev).clone()
         torch.cuda.synchronize()
         assert split.split_indices == [0, 12, 24]
-        assert rel_err(eager.float(), want) < TOL_BF16
-        for i in range(3):
-            manager.prepare(T, [1] * T, use_cudagraph=True)
-            y = compiled(*dev)
-            torch.cuda.synchronize()
-            assert torch.equal(y, eager), f"replay {i}"
-            torch.randn(128, 128, device="cuda").sum().item()
-    assert len(manager._schedule_graphs) == 1
-    # the caches hold the oracle's appended entries
-    from dynaflow_amd.decode import unpack_v_cache
+        assert rel_err(y.float(), want) < TOL_BF16
+        again = compiled_again(manager, compiled, dev, T)      # a decode step with fixed lengths is idempotent
+        assert torch.equal(again, y)
+    trace = manager.engine.issue_trace
+    assert trace[:3] == [(subs[0], 0), (subs[1], 0), (subs[0], 1)] and len(trace) == 12
     for i, blk in enumerate(model.attn):
         got_k = blk.k_cache.double().cpu().permute(0, 2, 1, 3)
         assert (got_k - kc[i]).abs().max() <= 0.05 * kc[i].abs().max()
+
+
+def compiled_again(manager, compiled, dev, T):
+    manager.prepare(T, [1] * T, use_cudagraph=False)
+    out = compiled(*dev)
+    torch.cuda.synchronize()
+    return out
+
+
+def test_whole_schedule_capture_of_many_sub_graphs_is_refused():
+    """Capturing the whole two-stream schedule of a multi-layer model (more than two sub-graphs per
+    nano-batch) ended in a segmentation fault inside stream capture on this runtime; the manager refuses
+    it instead (per-sub-graph graphs and the eager schedule remain)."""
+    T = 8
+    manager, compiled, dev, *_ = build_decode(T, whole_graph=True, layers=2)
+    with torch.no_grad():
+        manager.prepare(T, [1] * T, use_cudagraph=True)
+        with pytest.raises(NotImplementedError):
+            compiled(*dev)
 
 
 def test_decode_attention_under_graph_capture(ops):
