@@ -216,6 +216,14 @@ DFHIP_DEVICE f32x4 load_f32x4_device_coherent(const f32x4* p) {
 // be used after this, which ties the wait to the register so that the use cannot move above it.
 DFHIP_DEVICE void wait_loaded(f32x4& v) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(v)::"memory"); }
 
+// Split-K workspaces start with the arrival counters.  Both split-K kernels use the same size of
+// counter area for a workspace (at least 4 KiB), so that the fp32 blocks one of them leaves behind
+// never lie where the other expects counters that are zero.
+size_t counter_area(size_t tiles) {
+  const size_t need = ((tiles * sizeof(int)) + 255) & ~(size_t)255;
+  return need > 4096 ? need : 4096;
+}
+
 // FUSED = false: C[M,N] = A W^T.
 // FUSED = true : C[M,N] = silu(A W^T) * (A W2^T) with W = gate weight, W2 = up weight, N = the
 //   intermediate size.  A tile is 256 rows x 128 columns; its "W half" holds 128 gate rows and 128 up
@@ -495,8 +503,7 @@ int launch_ring(const void* A, int64_t lda, const void* W, const void* W2, int64
   int* arrivals = static_cast<int*>(workspace);
   float* partials = nullptr;
   if (split_k > 1) {
-    const size_t counter_bytes = (((size_t)tiles_m * tiles_n * sizeof(int)) + 255) & ~(size_t)255;
-    partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + counter_bytes);
+    partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + counter_area((size_t)tiles_m * tiles_n));
   }
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * split_k), dim3(RTHREADS), RING_LDS, stream,
                      static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W),
@@ -727,6 +734,187 @@ int launch_ring224(const void* A, int64_t lda, const void* W, const void* W2, in
   return dfhip_check_launch();
 }
 
+
+// ------------------------------------------------------------------ weight-streaming kernel, M <= 128
+// Decode-sized activations (one nano-batch of single-token queries): the GEMM is bound by reading W
+// once from HBM.  Tile 128 (all rows of A) x 128 columns, 4 waves of 64 x 64, K in slabs of 64 through
+// a ring of four 32 KiB units (A half + W half of a slab) filled by LDS-DMA, three slabs in flight per
+// workgroup.  K is split over `split_k` workgroups per tile so that about 256 workgroups stream
+// different parts of W at the same time; the parts meet through the same ticket scheme as above.
+// Workgroups of one K part are neighbours (they share the A columns of that part in one XCD's L2).
+constexpr int SK_BM = 128, SK_BN = 128, SK_UNITS = 4, SK_UNIT = 32768, SK_LDS = SK_UNITS * SK_UNIT;
+
+__global__ void __launch_bounds__(RTHREADS)
+gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, uint16_t* __restrict__ C,
+                        int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int tiles_n, int split_k,
+                        float* __restrict__ partials, int* __restrict__ arrivals) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave & 1, wave_n = wave >> 1;
+  const int work = remap_xcd(blockIdx.x, tiles_n * split_k);
+  const int part = work / tiles_n;
+  const int tile = work - part * tiles_n;
+  const int n0 = tile * SK_BN;
+  const int slabs_total = K / BK;
+  const int slab0 = (int)((int64_t)slabs_total * part / split_k);
+  const int KT = (int)((int64_t)slabs_total * (part + 1) / split_k) - slab0;
+
+  // DMA: a half is 128 rows x 128 bytes = 16 instructions of 8 rows, 4 per wave
+  const uint8_t* a_src[4];
+  const uint8_t* w_src[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int row = (wave * 4 + t) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    int ar = row < M ? row : M - 1;
+    int wr = n0 + row; wr = wr < N ? wr : N - 1;
+    a_src[t] = reinterpret_cast<const uint8_t*>(A + (int64_t)ar * lda + chunk * 8);
+    w_src[t] = reinterpret_cast<const uint8_t*>(W + (int64_t)wr * ldw + chunk * 8);
+  }
+  auto issue = [&](int slab, int unit) {
+    const int64_t off = (int64_t)(slab0 + (slab < KT ? slab : KT - 1)) * (BK * 2);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) dma16(unit * SK_UNIT + (wave * 4 + t) * 1024, a_src[t] + off);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) dma16(unit * SK_UNIT + 16384 + (wave * 4 + t) * 1024, w_src[t] + off);
+  };
+
+  const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
+  int koff[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) koff[ks] = ((2 * ks + fhalf) ^ fswz) * 16;
+  const int a_lane = (wave_m * 64 + frow) * 128, w_lane = 16384 + (wave_n * 64 + frow) * 128;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  issue(0, 0);
+  issue(1, 1);
+  issue(2, 2);
+  for (int kt = 0; kt < KT; ++kt) {
+    wait_vmcnt<16>();        // slab kt has landed; kt+1 and kt+2 may be in flight
+    workgroup_barrier();     // ... for every wave, and everybody is done with slab kt-1
+    issue(kt + 3, (kt + 3) % SK_UNITS);
+    const uint8_t* u = smem + (kt % SK_UNITS) * SK_UNIT;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      bf16x8 fa[2], fw[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(u + a_lane + i * 4096 + koff[ks]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) fw[j] = *reinterpret_cast<const bf16x8*>(u + w_lane + j * 4096 + koff[ks]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[j], fa[i], acc[i][j], 0, 0, 0);
+    }
+  }
+  wait_vmcnt<0>();
+  workgroup_barrier();
+
+  if (split_k > 1) {
+    f32x4* mine = reinterpret_cast<f32x4*>(partials) + ((int64_t)tile * split_k + part) * (16 * RTHREADS) + tid;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+          store_f32x4_device_coherent(mine + ((i * 2 + j) * 4 + g) * RTHREADS, v);
+        }
+    wait_vmcnt<0>();
+    __syncthreads();
+    int* ticket_cell = reinterpret_cast<int*>(smem);
+    if (tid == 0) *ticket_cell = atomicAdd(arrivals + tile, 1);
+    __syncthreads();
+    const int ticket = *ticket_cell;
+    __syncthreads();
+    if (ticket != split_k - 1) return;
+    if (tid == 0) atomicExch(arrivals + tile, 0);
+    // the last arriver adds the parts in part order (its own is read back like the others)
+    const f32x4* all = reinterpret_cast<const f32x4*>(partials) + (int64_t)tile * split_k * (16 * RTHREADS) + tid;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    for (int p = 0; p < split_k; ++p) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        f32x4 v[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) v[c] = load_f32x4_device_coherent(all + ((int64_t)p * 16 + h * 8 + c) * RTHREADS);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) wait_loaded(v[c]);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          const int i = h, j = c >> 2, g = c & 3;
+          acc[i][j][4 * g] += v[c][0];
+          acc[i][j][4 * g + 1] += v[c][1];
+          acc[i][j][4 * g + 2] += v[c][2];
+          acc[i][j][4 * g + 3] += v[c][3];
+        }
+      }
+    }
+  }
+
+  // park 64 rows x 64 columns per wave (144-byte rows), then whole 128-byte row pieces
+  constexpr int PROW = 144;
+  uint8_t* park = smem + wave * (64 * PROW);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 v;
+        v[0] = pack2_bf16(acc[i][j][4 * g + 0], acc[i][j][4 * g + 1]);
+        v[1] = pack2_bf16(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+        *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * PROW + (j * 32 + g * 8 + fhalf * 4) * 2) = v;
+      }
+  DFHIP_PIN;
+  const int m_base = wave_m * 64, n_base = n0 + wave_n * 64;
+#pragma unroll 4
+  for (int p = 0; p < 8; ++p) {
+    const int id = p * 64 + lane;
+    const int row = id >> 3, c = id & 7;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * PROW + c * 16);
+    const int m = m_base + row, n = n_base + c * 8;
+    if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+  }
+}
+
+size_t skinny_counter_bytes(int N) { return counter_area((size_t)(N + SK_BN - 1) / SK_BN); }
+
+int launch_skinny(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K,
+                  int split_k, void* workspace, hipStream_t stream) {
+  if (M > SK_BM) return DFHIP_ERR_BAD_SHAPE;
+  static bool lds_opted_in = false;
+  if (!lds_opted_in) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_skinny_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS) != hipSuccess)
+      return DFHIP_ERR_LAUNCH;
+    lds_opted_in = true;
+  }
+  const int tiles_n = (N + SK_BN - 1) / SK_BN;
+  int* arrivals = static_cast<int*>(workspace);
+  float* partials = nullptr;
+  if (split_k > 1) partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + skinny_counter_bytes(N));
+  hipLaunchKernelGGL(gemm_bf16_skinny_kernel, dim3(tiles_n * split_k), dim3(RTHREADS), SK_LDS, stream,
+                     static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W), static_cast<uint16_t*>(C), M,
+                     N, K, lda, ldw, ldc, tiles_n, split_k, partials, arrivals);
+  return dfhip_check_launch();
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 int launch(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
            int K, hipStream_t stream) {
@@ -779,6 +967,7 @@ extern "C" int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void
     case 2: return launch<128, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 3: return launch<256, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 5: return launch_ring224<false>(A, lda, W, nullptr, ldw, C, ldc, M, N, K, s);
+    case 6: return launch_skinny(A, lda, W, ldw, C, ldc, M, N, K, 1, nullptr, s);
     default: return DFHIP_ERR_BAD_ARGUMENT;
   }
 }
@@ -792,6 +981,17 @@ extern "C" int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* spli
   const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
   *variant = 2;
   *split_k = 1;
+  if (M <= SK_BM && M >= 16 && N >= 1024 && K >= 1024) {
+    // decode-sized activations: stream W with about 256 workgroups, at least 8 slabs per part
+    const int tiles_n = (N + SK_BN - 1) / SK_BN;
+    int s = (256 + tiles_n / 2) / tiles_n;
+    if (s < 1) s = 1;
+    if (s > 16) s = 16;
+    while (s > 1 && K / BK < 8 * s) --s;
+    *variant = 6;
+    *split_k = s;
+    return DFHIP_OK;
+  }
   if (M > 128 && N > 128 && big_tiles >= 32) {
     *variant = 0;
     int s = (int)(256 / big_tiles);
@@ -814,20 +1014,29 @@ extern "C" int dfhip_gemm_bf16_nt(const void* A, int64_t lda, const void* W, int
 extern "C" size_t dfhip_gemm_bf16_splitk_workspace_bytes(int M, int N, int split_k) {
   if (M < 1 || N < 1 || split_k < 2) return 0;
   const size_t tiles = (size_t)((M + RBM - 1) / RBM) * ((N + RBN - 1) / RBN);
-  const size_t counter_bytes = ((tiles * sizeof(int)) + 255) & ~(size_t)255;
-  return counter_bytes + tiles * split_k * (size_t)RBM * RBN * sizeof(float);
+  const size_t ring = counter_area(tiles) + tiles * split_k * (size_t)RBM * RBN * sizeof(float);
+  if (M > SK_BM) return ring;
+  // the weight-streaming kernel (M <= 128) has its own layout; a caller sizes for whichever is used
+  const size_t skinny = skinny_counter_bytes(N) +
+                        (size_t)((N + SK_BN - 1) / SK_BN) * split_k * (size_t)SK_BM * SK_BN * sizeof(float);
+  return ring > skinny ? ring : skinny;
 }
 
 extern "C" int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                                          int64_t ldc, int M, int N, int K, int split_k, void* workspace,
                                          size_t workspace_bytes, dfhip_stream_t stream) {
   if (int rc = check_args(A, lda, W, ldw, C, ldc, M, N, K)) return rc;
-  if (split_k < 1 || split_k > 8 || K / BK < split_k) return DFHIP_ERR_BAD_ARGUMENT;
+  if (split_k < 1 || split_k > 16 || K / BK < split_k) return DFHIP_ERR_BAD_ARGUMENT;
   if (split_k > 1) {
     if (!workspace) return DFHIP_ERR_NULL_POINTER;
     if (!dfhip_aligned16(workspace)) return DFHIP_ERR_BAD_ALIGNMENT;
     if (workspace_bytes < dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k)) return DFHIP_ERR_BAD_ARGUMENT;
   }
+  int variant = 0, planned = 1;
+  dfhip_gemm_bf16_plan(M, N, K, &variant, &planned);
+  if (variant == 6)
+    return launch_skinny(A, lda, W, ldw, C, ldc, M, N, K, split_k, workspace, static_cast<hipStream_t>(stream));
+  if (split_k > 8) return DFHIP_ERR_BAD_ARGUMENT;
   return launch_ring<false>(A, lda, W, nullptr, ldw, C, ldc, M, N, K, split_k, workspace,
                             static_cast<hipStream_t>(stream));
 }

@@ -67,6 +67,11 @@ class CUDAGraphWrapper:
             assert handle._is_dryrun, (
                 f"CUDA graph capture is required for batch size {size} but not in dry-run mode"
             )
+            # one eager call first: lazy one-time set-up (kernel attributes, split-K workspaces) must not
+            # happen under capture.  Sub-graphs that write state (a KV-cache append) write the same
+            # values again in the capture's replay below.
+            self.runnable(*args, **kwargs)
+            torch.cuda.current_stream().synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool=_global_pool.get_pool(handle.batch_idx)):
                 out = self.runnable(*args, **kwargs)

@@ -87,9 +87,15 @@ SPLIT_K_ENABLED = os.environ.get("DYNAFLOW_SPLIT_K", "1") != "0"
 def _splitk_workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
     key = (device.index or 0, stream)
     ws = _splitk_workspaces.get(key)
+    if torch.cuda.is_current_stream_capturing() and (ws is None or ws.numel() < nbytes):
+        # A capture on a stream of its own (per-sub-graph graphs): the workspace comes from the graph's
+        # memory pool and its counter area (at the start; 64 KiB are cleared) is zeroed by a fill kernel that is part of
+        # the graph - no memset node.  Graphs of one pool replay one after the other, so they may share.
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        rc = _cabi.load().dfhip_fill_u32(ws.data_ptr(), 0, min(nbytes, 65536) // 4, stream)
+        _cabi.check("dfhip_fill_u32", rc)
+        return ws
     if ws is None or ws.numel() < nbytes:
-        if torch.cuda.is_current_stream_capturing():
-            raise RuntimeError("split-K workspace must exist before graph capture: run the shape eagerly once")
         ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
         _splitk_workspaces[key] = ws
     return ws

@@ -120,7 +120,7 @@ def test_decode_attention_full_size_properties(ops):
     assert torch.equal(const, torch.full_like(const, 0.375))
 
 
-def build_decode(T, whole_graph, **over):
+def build_decode(T, whole_graph, sub_graphs=False, **over):
     from dynaflow_amd.backend import make_backend
     from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
     from dynaflow_amd.decode import DecodeModel
@@ -140,8 +140,9 @@ def build_decode(T, whole_graph, **over):
     slots = torch.randperm(cfg_model["slots"], generator=g)[:T].int()
     lengths = torch.randint(1, cfg_model["capacity"] + 1, (T,), generator=g).int()
     cfg = DynaFlowConfig("dynaflow_amd.schedulers:DecoderOverlapScheduler", 2, InductorConfig(enabled=True),
-                         CUDAGraphConfig(enabled=False, capture_sizes=[T]),
-                         {"min_nano_split_tokens": 1, "dump_graph": False, "whole_graph": whole_graph})
+                         CUDAGraphConfig(enabled=sub_graphs, capture_sizes=[T // 2, T]),
+                         {"min_nano_split_tokens": 1, "dump_graph": False, "whole_graph": whole_graph,
+                          "max_tokens": T})
     manager = DynaFlowManager()
     torch._dynamo.reset()
     dev = [t.cuda() for t in (ids, slots, lengths)]
@@ -239,3 +240,36 @@ def test_decode_attention_under_graph_capture(ops):
     torch.cuda.synchronize()
     want = ops.decode_attention(qkv, k_cache, v_cache, slots, lens, cos, sin, heads, kv_heads)
     assert torch.equal(out, want) and not torch.equal(out, eager)
+
+
+def test_decode_schedule_with_sub_graph_replay():
+    """Per-sub-graph graphs (the reference's mechanism) on the decode model at shapes where the projections
+    run on the weight-streaming kernel with K split: capture in a dry-run at the nano-batch size, then the
+    scheduled forward replays the graphs; every replay equals the eager two-stream result."""
+    T = 32
+    over = dict(layers=2, hidden=1024, heads=8, kv_heads=2, inter=2048)
+    print("decode sub-graph replay: eager model", flush=True)
+    manager, compiled, dev, host, model, inputs, cm = build_decode(T, whole_graph=False, **over)
+    with torch.no_grad():
+        manager.prepare(T, [1] * T)
+        eager = compiled(*dev).clone()
+        torch.cuda.synchronize()
+    print("decode sub-graph replay: graph model", flush=True)
+    manager, compiled, dev, host2, model2, _, _ = build_decode(T, whole_graph=False, sub_graphs=True, **over)
+    half = T // 2
+    with torch.no_grad():
+        print("decode sub-graph replay: dry-run capture", flush=True)
+        manager.prepare(half, [1] * half, is_dryrun=True, use_cudagraph=True)
+        compiled(*(t[:half].contiguous() for t in dev))
+        torch.cuda.synchronize()
+        for i in range(3):
+            print(f"decode sub-graph replay: replay {i}", flush=True)
+            split = manager.prepare(T, [1] * T, use_cudagraph=True)
+            assert split.use_cudagraph and split.num_tokens_padded == [half, half]
+            y = compiled(*dev)
+            torch.cuda.synchronize()
+            assert torch.equal(y, eager), f"replay {i}"
+            torch.randn(256, 256, device="cuda").sum().item()
+    names = [n.target for n in manager.graph_module.graph.nodes if n.op == "call_module"]
+    wrapper = manager.graph_module.__dict__[names[0]].callable_dynamic
+    assert sorted(k[:2] for k in wrapper._entries) == [(half, 0), (half, 1)]

@@ -331,3 +331,41 @@ def test_rope_against_complex_rotation(ops, B, S, heads, d):
     assert got.shape == t.shape
     assert bool(((got.float().cpu() - want.float()).abs() <= 2 ** -7 * want.float().abs() + 1e-6).all())
     assert torch.equal(got[:, 0].cpu(), t[:, 0])  # position 0 is the identity
+
+
+@pytest.mark.parametrize("M,N,K", [(7, 24, 64), (128, 128, 128), (50, 264, 192), (128, 1032, 320), (1, 8, 64)])
+def test_weight_streaming_gemm_small_shapes(ops, M, N, K):
+    a = randn((M, K), 1).bfloat16()
+    w = randn((N, K), 2, 0.05).bfloat16()
+    want = from_u16(cref.gemm_nt_bf16(u16(a), u16(w)))
+    got = ops.linear_variant(a.cuda(), w.cuda(), 6)
+    torch.cuda.synchronize()
+    g, w_ = got.float().cpu(), want.float()
+    assert got.shape == (M, N)
+    assert bool(((g - w_).abs() <= 2 ** -7 * w_.abs() + 2e-4 * w_.abs().max()).all())
+
+
+@pytest.mark.parametrize("M,N,K,split", [(128, 4096, 4096, 8), (100, 6144, 4096, 5), (128, 14336, 4096, 2),
+                                         (128, 4096, 14336, 8), (16, 1024, 1024, 2)])
+def test_weight_streaming_gemm_decode_shapes(ops, M, N, K, split):
+    """M <= 128: the plan picks the weight-streaming kernel and splits K so that about 256 workgroups stream W;
+    the parts are added in a fixed order, so the result is the same on every run."""
+    import ctypes
+
+    from dynaflow_amd import _cabi
+
+    lib = _cabi.load()
+    v, s = ctypes.c_int(), ctypes.c_int()
+    assert lib.dfhip_gemm_bf16_plan(M, N, K, ctypes.byref(v), ctypes.byref(s)) == 0
+    assert (v.value, s.value) == (6, split)
+    a = randn((M, K), 61).bfloat16().cuda()
+    w = randn((N, K), 62, 0.02).bfloat16().cuda()
+    got = ops.linear(a, w)
+    again = ops.linear(a, w)
+    whole = ops.linear_variant(a, w, -2)     # the same kernel, K not split
+    torch.cuda.synchronize()
+    assert torch.equal(got, again)
+    want = a.double().cpu() @ w.double().cpu().t()
+    assert rel_err(got.float(), want) < 2 ** -7 and rel_err(whole.float(), want) < 2 ** -7
+    g, w_ = got.float().cpu(), want.float()
+    assert bool(((g - w_).abs() <= 2 ** -7 * w_.abs() + 2e-4 * w_.abs().max()).all())
