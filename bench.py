@@ -318,7 +318,7 @@ def decode_config(torch, steps, warmup, layers=32):
     results = {}
     for name, knobs, graphs in (("serialized_eager", {"serialize": True}, False), ("overlapped_eager", {}, False),
                                 ("overlapped_sub_graph_replay", {}, True)):
-        extra = {"min_nano_split_tokens": 1, "dump_graph": False, "max_tokens": seqs}
+        extra = {"min_nano_split_tokens": 1, "dump_graph": False, "max_tokens": seqs, "fuse_silu_epilogue": True}
         extra.update(knobs)
         cfg = DynaFlowConfig("dynaflow_amd.schedulers:DecoderOverlapScheduler", 2, InductorConfig(enabled=True),
                              CUDAGraphConfig(enabled=graphs, capture_sizes=[half, seqs]), extra)

@@ -744,10 +744,16 @@ int launch_ring224(const void* A, int64_t lda, const void* W, const void* W2, in
 // Workgroups of one K part are neighbours (they share the A columns of that part in one XCD's L2).
 constexpr int SK_BM = 128, SK_BN = 128, SK_UNITS = 4, SK_UNIT = 32768, SK_LDS = SK_UNITS * SK_UNIT;
 
+// FUSED: C[M, N] = silu(A W^T) * (A W2^T) (gate and up weights, N = the intermediate size, K not split):
+// a tile is 128 rows x 64 columns, its W half holds, per wave column, 32 gate rows and the 32 matching up
+// rows, so MFMA block j = 0 is the gate and j = 1 the up projection of the same outputs.
+template <bool FUSED>
 __global__ void __launch_bounds__(RTHREADS)
-gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, uint16_t* __restrict__ C,
+gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
+                        const uint16_t* __restrict__ W2, uint16_t* __restrict__ C,
                         int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int tiles_n, int split_k,
                         float* __restrict__ partials, int* __restrict__ arrivals) {
+  constexpr int TILE_N = FUSED ? SK_BN / 2 : SK_BN;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -755,7 +761,7 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
   const int work = remap_xcd(blockIdx.x, tiles_n * split_k);
   const int part = work / tiles_n;
   const int tile = work - part * tiles_n;
-  const int n0 = tile * SK_BN;
+  const int n0 = tile * TILE_N;
   const int slabs_total = K / BK;
   const int slab0 = (int)((int64_t)slabs_total * part / split_k);
   const int KT = (int)((int64_t)slabs_total * (part + 1) / split_k) - slab0;
@@ -768,9 +774,15 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
     const int row = (wave * 4 + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     int ar = row < M ? row : M - 1;
-    int wr = n0 + row; wr = wr < N ? wr : N - 1;
     a_src[t] = reinterpret_cast<const uint8_t*>(A + (int64_t)ar * lda + chunk * 8);
-    w_src[t] = reinterpret_cast<const uint8_t*>(W + (int64_t)wr * ldw + chunk * 8);
+    if (FUSED) {
+      const int block = row >> 5;                       // 32-row block: wave column block/2, (0: gate, 1: up)
+      int wr = n0 + (block >> 1) * 32 + (row & 31); wr = wr < N ? wr : N - 1;
+      w_src[t] = reinterpret_cast<const uint8_t*>(((block & 1) ? W2 : W) + (int64_t)wr * ldw + chunk * 8);
+    } else {
+      int wr = n0 + row; wr = wr < N ? wr : N - 1;
+      w_src[t] = reinterpret_cast<const uint8_t*>(W + (int64_t)wr * ldw + chunk * 8);
+    }
   }
   auto issue = [&](int slab, int unit) {
     const int64_t off = (int64_t)(slab0 + (slab < KT ? slab : KT - 1)) * (BK * 2);
@@ -867,6 +879,39 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
     }
   }
 
+  if (FUSED) {
+    // the roundings of the separate kernels: bf16 projections, bf16 silu, bf16 product
+    constexpr int FROW = 80;
+    uint8_t* fpark = smem + wave * (64 * FROW);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float p[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][0][4 * g + e]));
+          const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][1][4 * g + e]));
+          p[e] = bf16_bits_to_f32(f32_to_bf16_bits(gt / (1.0f + expf(-gt)))) * ut;
+        }
+        u32x2 v;
+        v[0] = pack2_bf16(p[0], p[1]);
+        v[1] = pack2_bf16(p[2], p[3]);
+        *reinterpret_cast<u32x2*>(fpark + (i * 32 + frow) * FROW + (g * 8 + fhalf * 4) * 2) = v;
+      }
+    DFHIP_PIN;
+    const int fm_base = wave_m * 64, fn_base = n0 + wave_n * 32;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int id = p * 64 + lane;
+      const int row = id >> 2, c = id & 3;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(fpark + row * FROW + c * 16);
+      const int m = fm_base + row, n = fn_base + c * 8;
+      if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+    }
+    return;
+  }
+
   // park 64 rows x 64 columns per wave (144-byte rows), then whole 128-byte row pieces
   constexpr int PROW = 144;
   uint8_t* park = smem + wave * (64 * PROW);
@@ -895,23 +940,27 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
 
 size_t skinny_counter_bytes(int N) { return counter_area((size_t)(N + SK_BN - 1) / SK_BN); }
 
-int launch_skinny(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K,
-                  int split_k, void* workspace, hipStream_t stream) {
-  if (M > SK_BM) return DFHIP_ERR_BAD_SHAPE;
-  static bool lds_opted_in = false;
+template <bool FUSED>
+int launch_skinny(const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw, void* C, int64_t ldc, int M,
+                  int N, int K, int split_k, void* workspace, hipStream_t stream) {
+  if (M > SK_BM || (FUSED && split_k != 1)) return DFHIP_ERR_BAD_SHAPE;
+  auto kernel = gemm_bf16_skinny_kernel<FUSED>;
+  static bool lds_opted_in = false;   // one flag per instantiation
   if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_skinny_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, SK_LDS) != hipSuccess)
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            SK_LDS) != hipSuccess)
       return DFHIP_ERR_LAUNCH;
     lds_opted_in = true;
   }
-  const int tiles_n = (N + SK_BN - 1) / SK_BN;
+  constexpr int TILE_N = FUSED ? SK_BN / 2 : SK_BN;
+  const int tiles_n = (N + TILE_N - 1) / TILE_N;
   int* arrivals = static_cast<int*>(workspace);
   float* partials = nullptr;
   if (split_k > 1) partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + skinny_counter_bytes(N));
-  hipLaunchKernelGGL(gemm_bf16_skinny_kernel, dim3(tiles_n * split_k), dim3(RTHREADS), SK_LDS, stream,
-                     static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W), static_cast<uint16_t*>(C), M,
-                     N, K, lda, ldw, ldc, tiles_n, split_k, partials, arrivals);
+  hipLaunchKernelGGL(kernel, dim3(tiles_n * split_k), dim3(RTHREADS), SK_LDS, stream,
+                     static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W),
+                     static_cast<const uint16_t*>(W2), static_cast<uint16_t*>(C), M, N, K, lda, ldw, ldc, tiles_n,
+                     split_k, partials, arrivals);
   return dfhip_check_launch();
 }
 
@@ -967,7 +1016,7 @@ extern "C" int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void
     case 2: return launch<128, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 3: return launch<256, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 5: return launch_ring224<false>(A, lda, W, nullptr, ldw, C, ldc, M, N, K, s);
-    case 6: return launch_skinny(A, lda, W, ldw, C, ldc, M, N, K, 1, nullptr, s);
+    case 6: return launch_skinny<false>(A, lda, W, nullptr, ldw, C, ldc, M, N, K, 1, nullptr, s);
     default: return DFHIP_ERR_BAD_ARGUMENT;
   }
 }
@@ -1035,7 +1084,8 @@ extern "C" int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void*
   int variant = 0, planned = 1;
   dfhip_gemm_bf16_plan(M, N, K, &variant, &planned);
   if (variant == 6)
-    return launch_skinny(A, lda, W, ldw, C, ldc, M, N, K, split_k, workspace, static_cast<hipStream_t>(stream));
+    return launch_skinny<false>(A, lda, W, nullptr, ldw, C, ldc, M, N, K, split_k, workspace,
+                                static_cast<hipStream_t>(stream));
   if (split_k > 8) return DFHIP_ERR_BAD_ARGUMENT;
   return launch_ring<false>(A, lda, W, nullptr, ldw, C, ldc, M, N, K, split_k, workspace,
                             static_cast<hipStream_t>(stream));
@@ -1047,6 +1097,9 @@ extern "C" int dfhip_gemm_bf16_gate_up_silu(const void* A, int64_t lda, const vo
   if (!W_up) return DFHIP_ERR_NULL_POINTER;
   if (int rc = check_args(A, lda, W_gate, ldw, Out, ldo, M, I, K)) return rc;
   if (!dfhip_aligned16(W_up)) return DFHIP_ERR_BAD_ALIGNMENT;
+  if (M <= SK_BM && I >= 1024 && K >= 1024)   // decode-sized activations: stream both weights once
+    return launch_skinny<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, 1, nullptr,
+                               static_cast<hipStream_t>(stream));
   if (round_fill(M, I, TBN / 2) > round_fill(M, I, 128) + 0.05)
     return launch_ring224<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, static_cast<hipStream_t>(stream));
   return launch_ring<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, 1, nullptr,

@@ -284,18 +284,20 @@ def test_down_projection_shape_uses_split_k_and_matches_unsplit(ops):
 
 
 @pytest.mark.parametrize("M,I,K", [(1, 8, 64), (300, 264, 192), (257, 136, 128), (512, 1408, 512),
-                                   (2048, 14336, 128), (2000, 14328, 192)])
+                                   (2048, 14336, 128), (2000, 14328, 192), (128, 2048, 1024), (100, 1032, 1088)])
 def test_gate_up_silu_fused_epilogue(ops, M, I, K):
     """One launch for linear, linear, silu, mul.  The epilogue applies the roundings of the separate kernels,
     so the result has the same bits as linear, linear, silu_mul.  The two large shapes take the 256 x (112
     gate + 112 up) tile (I = 7 * 2^k fills the rounds of 256 workgroups), the others the 256 x (128 + 128)
-    tile; (2000, 14328) has ragged tiles in both directions."""
+    tile; (2000, 14328) has ragged tiles in both directions.  The last two (M <= 128) take the weight-streaming
+    kernel with both weights in one 128 x (32 gate + 32 up) x 2 tile."""
     x = randn((M, K), 41).bfloat16()
     wg = randn((I, K), 42, 0.05).bfloat16()
     wu = randn((I, K), 43, 0.05).bfloat16()
     got = ops.gate_up_silu(x.cuda(), wg.cuda(), wu.cuda())
     assert got.shape == (M, I) and got.dtype == torch.bfloat16
-    two = ops.silu_mul(ops.linear(x.cuda(), wg.cuda()), ops.linear(x.cuda(), wu.cuda()), True)
+    # (-2: the planned kernel with K not split - a split changes the order of the fp32 additions)
+    two = ops.silu_mul(ops.linear_variant(x.cuda(), wg.cuda(), -2), ops.linear_variant(x.cuda(), wu.cuda(), -2), True)
     assert torch.equal(got, two)
     # and against a float64 evaluation (three bf16 roundings; the one of the gate is amplified by
     # up to |1 + g(1 - sigmoid(g))| in silu)
