@@ -61,6 +61,8 @@ SIGNATURES: dict[str, tuple] = {
         c_int,
         [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, c_int, _P, c_size_t, _P],
     ),
+    "dfhip_gemm_bf16_nt_add": (c_int, [_P, c_int64, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_int, c_int, _P,
+                                       c_size_t, _P]),
     "dfhip_gemm_bf16_gate_up_silu": (c_int, [_P, c_int64, _P, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P]),
     "dfhip_gemm_f32_nt": (c_int, [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P]),
     "dfhip_gemm_fp8_nt": (

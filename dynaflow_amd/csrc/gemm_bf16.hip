@@ -57,11 +57,19 @@ struct Shape {
   static_assert((BM * CHUNKS) % THREADS == 0 && (BN * CHUNKS) % THREADS == 0, "loads must divide evenly");
 };
 
+// bf16(x + r) on packed pairs: the product is rounded to bf16 first (x is such a rounded value), the
+// sum is rounded again - the roundings of a GEMM followed by a separate bf16 addition.
+DFHIP_DEVICE uint32_t add2_bf16(uint32_t x, uint32_t r) {
+  return pack2_bf16(bf16_bits_to_f32(x & 0xffffu) + bf16_bits_to_f32(r & 0xffffu),
+                    __uint_as_float(x & 0xffff0000u) + __uint_as_float(r & 0xffff0000u));
+}
+
+// R (may be null): residual [M, N] with the leading dimension of C, added in the epilogue.
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_bf16_nt_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
-                    uint16_t* __restrict__ C, int M, int N, int K, int64_t lda, int64_t ldw,
-                    int64_t ldc, int tiles_m, int tiles_n) {
+                    const uint16_t* __restrict__ R, uint16_t* __restrict__ C, int M, int N, int K, int64_t lda,
+                    int64_t ldw, int64_t ldc, int tiles_m, int tiles_n) {
   using S = Shape<BM, BN, WAVES_M, WAVES_N>;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
@@ -187,6 +195,11 @@ gemm_bf16_nt_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
           u32x2 v;
           v[0] = pack2_bf16(acc[i][j][4 * g + 0], acc[i][j][4 * g + 1]);
           v[1] = pack2_bf16(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+          if (R) {
+            const u32x2 r = *reinterpret_cast<const u32x2*>(R + (int64_t)m * ldc + n);
+            v[0] = add2_bf16(v[0], r[0]);
+            v[1] = add2_bf16(v[1], r[1]);
+          }
           *reinterpret_cast<u32x2*>(c_row + n) = v;
         }
       }
@@ -480,9 +493,16 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   for (int p = 0; p < 32; ++p) {
     const int id = p * 64 + lane;
     const int row = id >> 4, c = id & 15;
-    const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * EROW + c * 16);
+    u32x4 v = *reinterpret_cast<const u32x4*>(park + row * EROW + c * 16);
     const int m = m_base + row, n = n_base + c * 8;
-    if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;  // N % 8 == 0
+    if (m < M && n < N) {  // N % 8 == 0
+      if (W2) {            // not FUSED: W2 is the optional residual [M, N] (leading dimension ldc)
+        const u32x4 r = *reinterpret_cast<const u32x4*>(W2 + (int64_t)m * ldc + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = add2_bf16(v[e], r[e]);
+      }
+      *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+    }
   }
 }
 
@@ -707,9 +727,16 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
   for (int p = 0; p < 28; ++p) {
     const int id = p * 64 + lane;
     const int row = id / 28, c = id - row * 28;
-    const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * TROW + c * 16);
+    u32x4 v = *reinterpret_cast<const u32x4*>(park + row * TROW + c * 16);
     const int m = m_base + row, n = n0 + c * 8;
-    if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+    if (m < M && n < N) {
+      if (W2) {            // not FUSED: W2 is the optional residual [M, N] (leading dimension ldc)
+        const u32x4 r = *reinterpret_cast<const u32x4*>(W2 + (int64_t)m * ldc + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = add2_bf16(v[e], r[e]);
+      }
+      *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+    }
   }
 }
 
@@ -932,9 +959,16 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
   for (int p = 0; p < 8; ++p) {
     const int id = p * 64 + lane;
     const int row = id >> 3, c = id & 7;
-    const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * PROW + c * 16);
+    u32x4 v = *reinterpret_cast<const u32x4*>(park + row * PROW + c * 16);
     const int m = m_base + row, n = n_base + c * 8;
-    if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+    if (m < M && n < N) {
+      if (W2) {            // not FUSED: W2 is the optional residual [M, N] (leading dimension ldc)
+        const u32x4 r = *reinterpret_cast<const u32x4*>(W2 + (int64_t)m * ldc + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = add2_bf16(v[e], r[e]);
+      }
+      *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+    }
   }
 }
 
@@ -966,7 +1000,7 @@ int launch_skinny(const void* A, int64_t lda, const void* W, const void* W2, int
 
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 int launch(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
-           int K, hipStream_t stream) {
+           int K, hipStream_t stream, const void* R = nullptr) {
   using S = Shape<BM, BN, WAVES_M, WAVES_N>;
   auto kernel = gemm_bf16_nt_kernel<BM, BN, WAVES_M, WAVES_N>;
   static bool lds_opted_in = false;  // attribute is per function, set once per process
@@ -980,7 +1014,8 @@ int launch(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int6
   const int tiles_n = (N + BN - 1) / BN;
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(S::THREADS), S::LDS_BYTES, stream,
                      static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W),
-                     static_cast<uint16_t*>(C), M, N, K, lda, ldw, ldc, tiles_m, tiles_n);
+                     static_cast<const uint16_t*>(R), static_cast<uint16_t*>(C), M, N, K, lda, ldw, ldc, tiles_m,
+                     tiles_n);
   return dfhip_check_launch();
 }
 
@@ -1104,4 +1139,29 @@ extern "C" int dfhip_gemm_bf16_gate_up_silu(const void* A, int64_t lda, const vo
     return launch_ring224<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, static_cast<hipStream_t>(stream));
   return launch_ring<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, 1, nullptr,
                            static_cast<hipStream_t>(stream));
+}
+
+extern "C" int dfhip_gemm_bf16_nt_add(const void* A, int64_t lda, const void* W, int64_t ldw, const void* R, void* C,
+                                      int64_t ldc, int M, int N, int K, int split_k, void* workspace,
+                                      size_t workspace_bytes, dfhip_stream_t stream) {
+  if (!R) return DFHIP_ERR_NULL_POINTER;
+  if (int rc = check_args(A, lda, W, ldw, C, ldc, M, N, K)) return rc;
+  if (!dfhip_aligned16(R)) return DFHIP_ERR_BAD_ALIGNMENT;
+  int variant = 2, planned = 1;
+  if (int rc = dfhip_gemm_bf16_plan(M, N, K, &variant, &planned)) return rc;
+  if (split_k < 1 || split_k > 16 || K / BK < split_k) return DFHIP_ERR_BAD_ARGUMENT;
+  if (split_k > 1) {
+    if (variant != 0 && variant != 6) return DFHIP_ERR_BAD_ARGUMENT;   // the planned kernel does not split K
+    if (variant == 0 && split_k > 8) return DFHIP_ERR_BAD_ARGUMENT;
+    if (!workspace) return DFHIP_ERR_NULL_POINTER;
+    if (!dfhip_aligned16(workspace)) return DFHIP_ERR_BAD_ALIGNMENT;
+    if (workspace_bytes < dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k)) return DFHIP_ERR_BAD_ARGUMENT;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (variant) {
+    case 0: return launch_ring<false>(A, lda, W, R, ldw, C, ldc, M, N, K, split_k, workspace, s);
+    case 5: return launch_ring224<false>(A, lda, W, R, ldw, C, ldc, M, N, K, s);
+    case 6: return launch_skinny<false>(A, lda, W, R, ldw, C, ldc, M, N, K, split_k, workspace, s);
+    default: return launch<128, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s, R);
+  }
 }

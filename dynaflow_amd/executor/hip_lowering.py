@@ -11,6 +11,9 @@ it deep-copies the sub-``GraphModule`` and replaces
 * ``attend_and_append(qkv, k_cache, v_cache, ...)``   -> ``dynaflow_hip.decode_attention``
 * ``causal_gqa_attention(q, k, v)`` (bf16, d 128, S%64) -> ``dynaflow_hip.causal_attention``
 
+* ``add(r, linear(x, w))`` (bf16, same shapes, the linear used once) -> ``dynaflow_hip.linear_add``
+  (the residual addition as the GEMM's epilogue; same roundings, same bits)
+
 With ``fuse_silu_epilogue`` a third rewrite follows: a ``silu_mul`` whose gate and up
 inputs are two bf16 ``linear`` nodes of the same activation becomes one
 ``dynaflow_hip.gate_up_silu(x, w_gate, w_up)`` - the SiLU*mul as the GEMM's epilogue.
@@ -218,6 +221,33 @@ def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False) -> tuple[
         node.replace_all_uses_with(new)
         graph.erase_node(node)
         stats["decode_attention"] = stats.get("decode_attention", 0) + 1
+
+    _ADD_TARGETS = {operator.add, torch.add}
+    for node in list(graph.nodes):
+        if node.op != "call_function" or node.target not in _ADD_TARGETS or len(node.args) != 2 or node.kwargs:
+            continue
+        for lin, other in ((node.args[1], node.args[0]), (node.args[0], node.args[1])):
+            if not isinstance(lin, fx.Node) or not isinstance(other, fx.Node):
+                continue
+            if lin.op != "call_function" or lin.target is not ops.linear or len(lin.users) != 1:
+                continue
+            el, eo = _example(lin), _example(other)
+            if not isinstance(el, torch.Tensor) or not isinstance(eo, torch.Tensor):
+                continue
+            if el.dtype != torch.bfloat16 or eo.dtype != torch.bfloat16 or el.dim() != eo.dim():
+                continue
+            # no broadcasting: every dimension equal as traced (a token dimension may be written as two
+            # different symbolic expressions of the same number; the operator checks the real shapes)
+            if any(_traced_int(a) != _traced_int(b) or _traced_int(a) is None for a, b in zip(el.shape, eo.shape)):
+                continue
+            with graph.inserting_before(node):
+                new = graph.call_function(ops.linear_add, (lin.args[0], lin.args[1], other))
+            new.meta = dict(node.meta)
+            node.replace_all_uses_with(new)
+            graph.erase_node(node)
+            graph.erase_node(lin)
+            stats["linear_add"] = stats.get("linear_add", 0) + 1
+            break
 
     if fuse_silu_epilogue:
         for node in list(graph.nodes):

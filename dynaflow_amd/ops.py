@@ -38,6 +38,7 @@ _lib.define("add_rms_norm(Tensor x, Tensor residual, Tensor weight, float eps) -
 _lib.define("transpose_weight(Tensor w) -> Tensor")
 _lib.define("rope(Tensor t, Tensor cos, Tensor sin) -> Tensor")
 _lib.define("causal_attention(Tensor q, Tensor k, Tensor v) -> Tensor")
+_lib.define("linear_add(Tensor x, Tensor weight, Tensor residual) -> Tensor")
 _lib.define(
     "decode_attention(Tensor qkv, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor slots, Tensor lengths, "
     "Tensor cos, Tensor sin, int q_heads, int kv_heads) -> Tensor"
@@ -162,6 +163,45 @@ _lib.impl("linear", lambda x, w: _linear_impl(x, w), "CUDA")
 _lib.impl("linear_variant", lambda x, w, v: _linear_impl(x, w, v), "CUDA")
 torch.library.register_fake("dynaflow_hip::linear", _linear_fake, lib=_lib)
 torch.library.register_fake("dynaflow_hip::linear_variant", lambda x, w, v: _linear_fake(x, w), lib=_lib)
+
+
+# ------------------------------------------------ projection + residual addition
+def _linear_add_impl(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+    """``residual + x @ weight.T`` (bf16) in one launch, rounded like the separate linear and add kernels."""
+    _require_device(x, weight, residual)
+    lib = _cabi.load()
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or residual.dtype != torch.bfloat16:
+        raise RuntimeError("linear_add: bf16 tensors expected")
+    if weight.dim() != 2 or x.shape[-1] != weight.shape[1]:
+        raise RuntimeError(f"linear_add: x[..., {x.shape[-1]}] does not match weight {tuple(weight.shape)}")
+    a, M, K, lda = _rows(x)
+    w, N, _, ldw = _rows(weight)
+    if tuple(residual.shape) != (*x.shape[:-1], N):
+        raise RuntimeError(f"linear_add: residual {tuple(residual.shape)} does not match the output")
+    r = residual.reshape(M, N)
+    if r.stride(1) != 1 or r.stride(0) != N:
+        r = r.contiguous()
+    out = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    if M > 0:
+        stream = _stream()
+        _, split_k = _plan_bf16(lib, M, N, K)
+        ws_ptr, ws_bytes = 0, 0
+        if split_k > 1 and SPLIT_K_ENABLED:
+            nbytes = lib.dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k)
+            ws = _splitk_workspace(x.device, stream, nbytes)
+            ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
+        else:
+            split_k = 1
+        rc = lib.dfhip_gemm_bf16_nt_add(
+            a.data_ptr(), lda, w.data_ptr(), ldw, r.data_ptr(), out.data_ptr(), N, M, N, K, split_k, ws_ptr,
+            ws_bytes, stream,
+        )
+        _cabi.check("dfhip_gemm_bf16_nt_add", rc)
+    return out.view(*x.shape[:-1], N)
+
+
+_lib.impl("linear_add", _linear_add_impl, "CUDA")
+torch.library.register_fake("dynaflow_hip::linear_add", lambda x, w, r: _linear_fake(x, w), lib=_lib)
 
 
 # ------------------------------------------- gate/up projection + SiLU*mul epilogue
@@ -508,6 +548,7 @@ transpose_weight = torch.ops.dynaflow_hip.transpose_weight
 rope = torch.ops.dynaflow_hip.rope
 decode_attention = torch.ops.dynaflow_hip.decode_attention
 causal_attention = torch.ops.dynaflow_hip.causal_attention
+linear_add = torch.ops.dynaflow_hip.linear_add
 quant_fp8 = torch.ops.dynaflow_hip.quant_fp8
 silu_mul_quant_fp8 = torch.ops.dynaflow_hip.silu_mul_quant_fp8
 linear_fp8 = torch.ops.dynaflow_hip.linear_fp8

@@ -110,6 +110,16 @@ int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void* W, int64_t
                               int64_t ldc, int M, int N, int K, int split_k, void* workspace,
                               size_t workspace_bytes, dfhip_stream_t stream);
 
+/* C[M,N] = bf16( bf16(A W^T) + R ): the contraction with the residual addition
+ * that follows it in a decoder layer (FX nodes linear, add) as the epilogue of the
+ * kernel dfhip_gemm_bf16_plan picks.  R is [M,N] with the leading dimension of C;
+ * the roundings are those of the separate linear and add kernels, so the bits are
+ * the same.  split_k and workspace as in dfhip_gemm_bf16_nt_splitk (split_k = 1:
+ * workspace may be null). */
+int dfhip_gemm_bf16_nt_add(const void* A, int64_t lda, const void* W, int64_t ldw, const void* R, void* C,
+                           int64_t ldc, int M, int N, int K, int split_k, void* workspace,
+                           size_t workspace_bytes, dfhip_stream_t stream);
+
 /* Gate and up projection with the SiLU*mul as the GEMM's epilogue:
  *   Out[M,I] = bf16( silu(A W_gate^T) * (A W_up^T) )
  * - the FX nodes linear, linear, silu, mul of the MLP in one launch.  Both

@@ -371,3 +371,18 @@ def test_weight_streaming_gemm_decode_shapes(ops, M, N, K, split):
     assert rel_err(got.float(), want) < 2 ** -7 and rel_err(whole.float(), want) < 2 ** -7
     g, w_ = got.float().cpu(), want.float()
     assert bool(((g - w_).abs() <= 2 ** -7 * w_.abs() + 2e-4 * w_.abs().max()).all())
+
+
+@pytest.mark.parametrize("M,N,K", [(300, 264, 192), (7, 24, 64), (2048, 14336, 256), (2048, 4096, 256),
+                                   (2048, 4096, 2048), (128, 4096, 4096), (100, 1032, 1088), (2000, 14328, 192)])
+def test_linear_with_residual_epilogue(ops, M, N, K):
+    """linear + add in one launch on every kernel the plan can pick (small tile, ring with and without split-K,
+    256 x 224 tile, weight-streaming): the epilogue rounds like the two separate kernels, so the bits match."""
+    x = randn((M, K), 71).bfloat16().cuda()
+    w = randn((N, K), 72, 0.05).bfloat16().cuda()
+    r = randn((M, N), 73).bfloat16().cuda()
+    got = ops.linear_add(x, w, r)
+    want = r + ops.linear(x, w)
+    torch.cuda.synchronize()
+    assert got.shape == (M, N) and torch.equal(got, want)
+    assert torch.equal(ops.linear_add(x, w, r), got)      # run-to-run

@@ -365,10 +365,12 @@ def test_decoder_layer_attention_beside_mlp_small():
     names = [n.target for n in manager.graph_module.graph.nodes if n.op == "call_module"]
     mlp_graph = manager.graph_module.__dict__[names[1]].callable_dynamic
     targets = [n.target for n in mlp_graph.graph.nodes if n.op == "call_function"]
-    assert ops.rms_norm in targets and ops.silu_mul in targets and targets.count(ops.linear) == 3
+    assert ops.rms_norm in targets and ops.silu_mul in targets
+    assert targets.count(ops.linear) == 2 and targets.count(ops.linear_add) == 1   # down projection + residual
     attn_targets = [n.target for n in manager.graph_module.__dict__[names[0]].callable_dynamic.graph.nodes
                     if n.op == "call_function"]
-    assert attn_targets.count(ops.linear) == 4 and ops.rms_norm in attn_targets
+    assert attn_targets.count(ops.linear) == 3 and attn_targets.count(ops.linear_add) == 1
+    assert ops.rms_norm in attn_targets
     assert attn_targets.count(ops.rope) == 2
     with torch.no_grad():
         split = manager.prepare(batch, [S] * batch)
