@@ -405,6 +405,194 @@ int launch_fp8_ring(const void* A, int64_t lda, const void* W, int64_t ldw, void
   return dfhip_check_launch();
 }
 
+
+// ------------------------------------------------------------------ fp8 ring kernel, 256 x 224 tile
+// The same ring with 4 waves stacked along M, each 64 x 224 = 2 x 7 MFMA blocks: column counts of
+// the form 7 * 2^k (28672 = 128 * 224) then fill the rounds of 256 workgroups exactly.
+constexpr int F8_TBN = 224, F8_TROW = F8_TBN * 2 + 16;
+
+__global__ void __launch_bounds__(256)
+gemm_fp8_ring224_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, uint16_t* __restrict__ C,
+                        const float* __restrict__ a_scale, const float* __restrict__ w_scale, int M, int N, int K,
+                        int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  const int tile = remap_xcd(blockIdx.x, tiles_m * tiles_n);
+  const int per_panel = F8_GROUP_M * tiles_n;
+  const int first_m = (tile / per_panel) * F8_GROUP_M;
+  const int rows_in_panel = (tiles_m - first_m) < F8_GROUP_M ? (tiles_m - first_m) : F8_GROUP_M;
+  const int in_panel = tile % per_panel;
+  const int m0 = (first_m + in_panel % rows_in_panel) * 256;
+  const int n0 = (in_panel / rows_in_panel) * F8_TBN;
+  const int KT = K / FBK;
+
+  const uint8_t* a_src[8];
+  const uint8_t* w_src[7];
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    const int row = (wave * 8 + t) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    int ar = m0 + row; ar = ar < M ? ar : M - 1;
+    a_src[t] = A + (int64_t)ar * lda + chunk * 16;
+  }
+#pragma unroll
+  for (int t = 0; t < 7; ++t) {
+    const int row = (wave * 7 + t) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    int wr = n0 + row; wr = wr < N ? wr : N - 1;
+    w_src[t] = W + (int64_t)wr * ldw + chunk * 16;
+  }
+  auto dma_a = [&](int t, int slab, int unit) {
+    const int s = slab < KT ? slab : KT - 1;
+    dma16(unit * F8_UNIT + (wave * 8 + t) * 1024, a_src[t] + (int64_t)s * FBK);
+  };
+  auto dma_w = [&](int t, int slab, int unit) {
+    const int s = slab < KT ? slab : KT - 1;
+    dma16(unit * F8_UNIT + (wave * 7 + t) * 1024, w_src[t] + (int64_t)s * FBK);
+  };
+
+  const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
+  int koff[2][2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    koff[ks][0] = ((4 * ks + 2 * fhalf) ^ fswz) * 16;
+    koff[ks][1] = ((4 * ks + 2 * fhalf + 1) ^ fswz) * 16;
+  }
+  const int a_lane = (wave * 64 + frow) * 128, w_lane = frow * 128;
+
+  f32x16 acc[2][7];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 7; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_a(t, 0, 0);
+#pragma unroll
+  for (int t = 0; t < 7; ++t) dma_w(t, 0, 1);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_a(t, 1, 2);
+#pragma unroll
+  for (int t = 0; t < 7; ++t) dma_w(t, 1, 3);
+  wait_vmcnt<15>();
+  workgroup_barrier();
+
+  u32x4 fa[2][2][2], fw[2][7][2];   // [slot][block][low/high 16 bytes]
+  // 18 fragment halves in the order the MFMAs need them: A block 0, W blocks 0..6, A block 1
+  auto read_half = [&](int r, int ks, int slot, int unit_a, int unit_w) {
+    const int f = r >> 1, part = r & 1;
+    if (f == 0 || f == 8) {
+      const int i = f >> 3;
+      fa[slot][i][part] = *reinterpret_cast<const u32x4*>(smem + unit_a * F8_UNIT + a_lane + koff[ks][part] + i * 4096);
+    } else {
+      fw[slot][f - 1][part] =
+          *reinterpret_cast<const u32x4*>(smem + unit_w * F8_UNIT + w_lane + koff[ks][part] + (f - 1) * 4096);
+    }
+  };
+  auto mfma = [&](int q, int slot) {
+    const int i = q / 7, j = q % 7;
+    const i32x8 av = {(int)fa[slot][i][0][0], (int)fa[slot][i][0][1], (int)fa[slot][i][0][2], (int)fa[slot][i][0][3],
+                      (int)fa[slot][i][1][0], (int)fa[slot][i][1][1], (int)fa[slot][i][1][2], (int)fa[slot][i][1][3]};
+    const i32x8 wv = {(int)fw[slot][j][0][0], (int)fw[slot][j][0][1], (int)fw[slot][j][0][2], (int)fw[slot][j][0][3],
+                      (int)fw[slot][j][1][0], (int)fw[slot][j][1][1], (int)fw[slot][j][1][2], (int)fw[slot][j][1][3]};
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wv, av, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+  };
+
+  int ua = 0, uw = 1, ia = 4, iw = 0;
+#pragma unroll
+  for (int r = 0; r < 18; ++r) read_half(r, 0, 0, ua, uw);
+  for (int kt = 0; kt < KT; ++kt) {
+    // k-step 0: 18 fragment halves of step 1, then the 8 DMA instructions of A(kt+2): 26 side operations
+    // behind 14 MFMAs (two behind each of the first twelve)
+#pragma unroll
+    for (int q = 0; q < 14; ++q) {
+      mfma(q, 0);
+      const int first = q < 12 ? 2 * q : 12 + q, last = q < 11 ? 2 * q + 2 : 13 + q;
+#pragma unroll
+      for (int op = first; op < last; ++op) {
+        if (op < 18) read_half(op, 1, 1, ua, uw); else dma_a(op - 18, kt + 2, ia);
+      }
+      DFHIP_PIN;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    wait_vmcnt<8>();
+    workgroup_barrier();
+    int na = ua + 2; if (na >= F8_NUNITS) na -= F8_NUNITS;
+    int nw = uw + 2; if (nw >= F8_NUNITS) nw -= F8_NUNITS;
+    // k-step 1: the 7 DMA instructions of W(kt+2), then the 18 fragment halves of slab kt+1, step 0
+#pragma unroll
+    for (int q = 0; q < 14; ++q) {
+      mfma(q, 1);
+      const int first = q < 11 ? 2 * q : 11 + q, last = q < 10 ? 2 * q + 2 : 12 + q;
+#pragma unroll
+      for (int op = first; op < last; ++op) {
+        if (op < 7) dma_w(op, kt + 2, iw); else read_half(op - 7, 0, 0, na, nw);
+      }
+      DFHIP_PIN;
+    }
+    ua = na; uw = nw;
+    ia += 2; if (ia >= F8_NUNITS) ia -= F8_NUNITS;
+    iw += 2; if (iw >= F8_NUNITS) iw -= F8_NUNITS;
+  }
+  wait_vmcnt<0>();
+  workgroup_barrier();
+
+  const float sa = a_scale[0];
+  uint8_t* park = smem + wave * (64 * F8_TROW);
+#pragma unroll
+  for (int j = 0; j < 7; ++j)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      int n = n0 + j * 32 + g * 8 + fhalf * 4;
+      n = n < N ? n : N - 4;
+      const f32x4 ws = *reinterpret_cast<const f32x4*>(w_scale + n);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        u32x2 v;
+        v[0] = pack2_bf16(acc[i][j][4 * g + 0] * (sa * ws[0]), acc[i][j][4 * g + 1] * (sa * ws[1]));
+        v[1] = pack2_bf16(acc[i][j][4 * g + 2] * (sa * ws[2]), acc[i][j][4 * g + 3] * (sa * ws[3]));
+        *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * F8_TROW + (j * 32 + g * 8 + fhalf * 4) * 2) = v;
+      }
+    }
+  DFHIP_PIN;
+  const int m_base = m0 + wave * 64;
+#pragma unroll 4
+  for (int p = 0; p < 28; ++p) {
+    const int id = p * 64 + lane;
+    const int row = id / 28, c = id - row * 28;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * F8_TROW + c * 16);
+    const int m = m_base + row, n = n0 + c * 8;
+    if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+  }
+}
+
+int launch_fp8_ring224(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
+                       const float* a_scale, const float* w_scale, int M, int N, int K, hipStream_t stream) {
+  static bool lds_opted_in = false;
+  if (!lds_opted_in) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fp8_ring224_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, F8_RING_LDS) != hipSuccess)
+      return DFHIP_ERR_LAUNCH;
+    lds_opted_in = true;
+  }
+  const int tiles_m = (M + 255) / 256, tiles_n = (N + F8_TBN - 1) / F8_TBN;
+  hipLaunchKernelGGL(gemm_fp8_ring224_kernel, dim3(tiles_m * tiles_n), dim3(256), F8_RING_LDS, stream,
+                     static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(W), static_cast<uint16_t*>(C),
+                     a_scale, w_scale, M, N, K, lda, ldw, ldc, tiles_m, tiles_n);
+  return dfhip_check_launch();
+}
+
+// Fraction of the CU-rounds that do work when [M, N] is cut into 256 x tile_n tiles dealt to 256 CUs in rounds.
+double fp8_round_fill(int M, int N, int tile_n) {
+  const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + tile_n - 1) / tile_n);
+  const int64_t rounds = (tiles + 255) / 256;
+  return (double)M * N / ((double)rounds * 256 * 256 * tile_n);
+}
+
 template <int BM, int BN>
 int launch_fp8(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, const float* a_scale,
                const float* w_scale, int M, int N, int K, hipStream_t stream) {
@@ -478,9 +666,9 @@ extern "C" int dfhip_silu_mul_absmax_bf16(const void* gate, int64_t ld_gate, con
   return dfhip_check_launch();
 }
 
-extern "C" int dfhip_gemm_fp8_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
-                                 const float* a_scale, const float* w_scale, int M, int N, int K,
-                                 dfhip_stream_t stream) {
+extern "C" int dfhip_gemm_fp8_nt_variant(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                                         int64_t ldc, const float* a_scale, const float* w_scale, int M, int N,
+                                         int K, int variant, dfhip_stream_t stream) {
   if (!A || !W || !C || !a_scale || !w_scale) return DFHIP_ERR_NULL_POINTER;
   if (M < 1 || N < 1 || K < 1 || K % FBK != 0 || N % 8 != 0) return DFHIP_ERR_BAD_SHAPE;
   if (lda < K || ldw < K || ldc < N) return DFHIP_ERR_BAD_STRIDE;
@@ -488,8 +676,22 @@ extern "C" int dfhip_gemm_fp8_nt(const void* A, int64_t lda, const void* W, int6
       !dfhip_aligned16(w_scale))
     return DFHIP_ERR_BAD_ALIGNMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-  if (M > 128 && N > 128 && big_tiles >= 32)
-    return launch_fp8_ring(A, lda, W, ldw, C, ldc, a_scale, w_scale, M, N, K, s);
-  return launch_fp8<128, 128>(A, lda, W, ldw, C, ldc, a_scale, w_scale, M, N, K, s);
+  if (variant < 0) {   // the planned kernel
+    const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+    variant = 1;
+    if (M > 128 && N > 128 && big_tiles >= 32)
+      variant = fp8_round_fill(M, N, F8_TBN) > fp8_round_fill(M, N, 256) + 0.05 ? 2 : 0;
+  }
+  switch (variant) {
+    case 0: return launch_fp8_ring(A, lda, W, ldw, C, ldc, a_scale, w_scale, M, N, K, s);
+    case 1: return launch_fp8<128, 128>(A, lda, W, ldw, C, ldc, a_scale, w_scale, M, N, K, s);
+    case 2: return launch_fp8_ring224(A, lda, W, ldw, C, ldc, a_scale, w_scale, M, N, K, s);
+    default: return DFHIP_ERR_BAD_ARGUMENT;
+  }
+}
+
+extern "C" int dfhip_gemm_fp8_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
+                                 const float* a_scale, const float* w_scale, int M, int N, int K,
+                                 dfhip_stream_t stream) {
+  return dfhip_gemm_fp8_nt_variant(A, lda, W, ldw, C, ldc, a_scale, w_scale, M, N, K, -1, stream);
 }

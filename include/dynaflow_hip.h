@@ -145,6 +145,12 @@ int dfhip_gemm_f32_nt(const void* A, int64_t lda, const void* W, int64_t ldw, vo
 int dfhip_gemm_fp8_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                       int64_t ldc, const float* a_scale, const float* w_scale, int M, int N,
                       int K, dfhip_stream_t stream);
+/* The same with an explicit kernel, for tuning and tests: 0 = 256x256 LDS-DMA ring,
+ * 1 = register-staged 128x128, 2 = 256x224 LDS-DMA ring (N = 7 * 2^k), negative =
+ * the choice dfhip_gemm_fp8_nt makes. */
+int dfhip_gemm_fp8_nt_variant(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
+                              const float* a_scale, const float* w_scale, int M, int N, int K, int variant,
+                              dfhip_stream_t stream);
 
 /* ------------------------------------------------------------ elementwise
  *

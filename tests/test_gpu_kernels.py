@@ -386,3 +386,19 @@ def test_linear_with_residual_epilogue(ops, M, N, K):
     torch.cuda.synchronize()
     assert got.shape == (M, N) and torch.equal(got, want)
     assert torch.equal(ops.linear_add(x, w, r), got)      # run-to-run
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 8, 128), (300, 264, 384), (512, 1032, 1024), (2048, 3584, 256), (1100, 2056, 384)])
+@pytest.mark.parametrize("variant", [0, 1, 2])
+def test_gemm_fp8_variants_agree(ops, M, N, K, variant):
+    """Every fp8 kernel (256x256 ring, register-staged 128x128, 256x224 ring) on the same operands: products of
+    e4m3 values are exact in fp32 and all kernels add them in the same order, so the results are bit-identical."""
+    x = randn((M, K), 20).bfloat16()
+    w = randn((N, K), 21, 0.02).bfloat16()
+    xq, xs = mlp.quant_e4m3(x)
+    wq, ws = mlp.quant_e4m3_per_channel(w)
+    args = (xq.cuda().view(torch.float8_e4m3fn), wq.cuda().view(torch.float8_e4m3fn), xs.cuda(), ws.cuda())
+    got = ops.linear_fp8_variant(*args, variant)
+    want = mlp.dequant(xq, xs) @ mlp.dequant(wq, ws).t()
+    assert got.shape == (M, N) and rel_err(got.float(), want) < 2 ** -7
+    assert torch.equal(got, ops.linear_fp8_variant(*args, 1))
