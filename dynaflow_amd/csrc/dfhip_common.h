@@ -34,6 +34,12 @@ DFHIP_DEVICE uint32_t pack2_bf16(float lo, float hi) {
   return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
 }
 
+// silu(g) = g / (1 + e^-g) on the hardware exponential and reciprocal (a few fp32 ulp; the bf16 paths
+// round the result to 8 bits of mantissa right after).  -inf gives NaN like the exact quotient.
+DFHIP_DEVICE float silu_fast(float g) {
+  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
+}
+
 // 64-lane reductions through DPP-free shuffles (wave64)
 DFHIP_DEVICE float wave_sum(float v) {
 #pragma unroll

@@ -41,7 +41,7 @@ silu_mul_bf16_kernel(const uint16_t* __restrict__ gate, int64_t ld_gate, const u
     for (int w = 0; w < 4; ++w) {
       float g_lo = bf16_bits_to_f32(g[p][w] & 0xffffu), g_hi = __uint_as_float(g[p][w] & 0xffff0000u);
       float u_lo = bf16_bits_to_f32(u[p][w] & 0xffffu), u_hi = __uint_as_float(u[p][w] & 0xffff0000u);
-      float s_lo = silu_f32(g_lo), s_hi = silu_f32(g_hi);
+      float s_lo = silu_fast(g_lo), s_hi = silu_fast(g_hi);   // same formula as the GEMM epilogues: same bits
       if (ROUND_SILU) {
         s_lo = bf16_bits_to_f32(f32_to_bf16_bits(s_lo));
         s_hi = bf16_bits_to_f32(f32_to_bf16_bits(s_hi));

@@ -22,7 +22,7 @@ constexpr float FP8_MAX = 448.0f;
 constexpr int QT = 256;      // threads of the elementwise fp8 kernels
 constexpr int QUNROLL = 4;
 
-DFHIP_DEVICE float silu_f32(float g) { return g / (1.0f + expf(-g)); }
+DFHIP_DEVICE float silu_f32(float g) { return silu_fast(g); }   // one formula for every bf16 path
 
 DFHIP_DEVICE void atomic_max_nonneg(float* cell, float v) {
   // non-negative floats order like their bit patterns

@@ -457,7 +457,7 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
             // the roundings of the two-kernel path: bf16 projections, bf16 silu, bf16 product
             const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][4 * g + e]));
             const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j + 2][4 * g + e]));
-            p[e] = bf16_bits_to_f32(f32_to_bf16_bits(gt / (1.0f + expf(-gt)))) * ut;
+            p[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
           }
           u32x2 v;
           v[0] = pack2_bf16(p[0], p[1]);
@@ -716,8 +716,8 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
       for (int w = 0; w < 4; ++w) {
         const float g0 = bf16_bits_to_f32(g[w] & 0xffffu), g1 = __uint_as_float(g[w] & 0xffff0000u);
         const float u0 = bf16_bits_to_f32(u[w] & 0xffffu), u1 = __uint_as_float(u[w] & 0xffff0000u);
-        const float s0 = bf16_bits_to_f32(f32_to_bf16_bits(g0 / (1.0f + expf(-g0))));
-        const float s1 = bf16_bits_to_f32(f32_to_bf16_bits(g1 / (1.0f + expf(-g1))));
+        const float s0 = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(g0)));
+        const float s1 = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(g1)));
         v[w] = pack2_bf16(s0 * u0, s1 * u1);
       }
       const int m = m_base + row, n = n0 + c * 8;
@@ -921,7 +921,7 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
         for (int e = 0; e < 4; ++e) {
           const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][0][4 * g + e]));
           const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][1][4 * g + e]));
-          p[e] = bf16_bits_to_f32(f32_to_bf16_bits(gt / (1.0f + expf(-gt)))) * ut;
+          p[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
         }
         u32x2 v;
         v[0] = pack2_bf16(p[0], p[1]);
