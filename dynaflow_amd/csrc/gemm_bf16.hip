@@ -768,7 +768,7 @@ int launch_ring224(const void* A, int64_t lda, const void* W, const void* W2, in
 // Decode-sized activations (one nano-batch of single-token queries): the GEMM is bound by reading W
 // once from HBM.  Tile 128 (all rows of A) x 128 columns, 4 waves of 64 x 64, K in slabs of 64 through
 // a ring of four 32 KiB units (A half + W half of a slab) filled by LDS-DMA, three slabs in flight per
-// workgroup.  K is split over `split_k` workgroups per tile so that about 256 workgroups stream
+// workgroup.  K is split over `split_k` workgroups per tile so that about 200 workgroups stream
 // different parts of W at the same time; the parts meet through the same ticket scheme as above.
 // Workgroups of one K part are neighbours (they share the A columns of that part in one XCD's L2).
 constexpr int SK_BM = 128, SK_BN = 128, SK_UNITS = 4, SK_UNIT = 32768, SK_LDS = SK_UNITS * SK_UNIT;
@@ -835,27 +835,39 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
+  // Fragments are double-buffered by hand: the reads of k-step s+1 (or of the next slab's first k-step)
+  // are issued before the MFMAs of step s, so no LDS latency is exposed inside a slab or across slabs.
+  bf16x8 fa[2][2], fw[2][2];
+  auto read_frags = [&](int slab, int ks, int slot) {
+    const uint8_t* u = smem + (slab % SK_UNITS) * SK_UNIT;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) fa[slot][i] = *reinterpret_cast<const bf16x8*>(u + a_lane + i * 4096 + koff[ks]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) fw[slot][j] = *reinterpret_cast<const bf16x8*>(u + w_lane + j * 4096 + koff[ks]);
+  };
   issue(0, 0);
   issue(1, 1);
   issue(2, 2);
+  wait_vmcnt<8>();           // slabs 0 and 1 have landed
+  workgroup_barrier();
+  read_frags(0, 0, 0);
   for (int kt = 0; kt < KT; ++kt) {
-    wait_vmcnt<16>();        // slab kt has landed; kt+1 and kt+2 may be in flight
-    workgroup_barrier();     // ... for every wave, and everybody is done with slab kt-1
-    issue(kt + 3, (kt + 3) % SK_UNITS);
-    const uint8_t* u = smem + (kt % SK_UNITS) * SK_UNIT;
+    issue(kt + 3, (kt + 3) % SK_UNITS);   // into the unit of slab kt-1: everybody passed the barrier after it
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      bf16x8 fa[2], fw[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(u + a_lane + i * 4096 + koff[ks]);
-#pragma unroll
-      for (int j = 0; j < 2; ++j) fw[j] = *reinterpret_cast<const bf16x8*>(u + w_lane + j * 4096 + koff[ks]);
+      const int slot = ks & 1;
+      if (ks < 3) read_frags(kt, ks + 1, slot ^ 1); else read_frags(kt + 1, 0, slot ^ 1);   // slab kt+1 has landed
+      DFHIP_PIN;
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[j], fa[i], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
+      DFHIP_PIN;
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // every read of slab kt (and the prefetch) has returned
+    wait_vmcnt<8>();         // slab kt+2 has landed; only slab kt+3 may be in flight
+    workgroup_barrier();
   }
   wait_vmcnt<0>();
   workgroup_barrier();
@@ -1068,9 +1080,10 @@ extern "C" int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* spli
   *variant = 2;
   *split_k = 1;
   if (M <= SK_BM && M >= 16 && N >= 1024 && K >= 1024) {
-    // decode-sized activations: stream W with about 256 workgroups, at least 8 slabs per part
+    // decode-sized activations: stream W with about 192 workgroups (measured best over the 8B shapes: more
+    // parts shorten every workgroup's loop below its fixed costs), at least 8 slabs per part
     const int tiles_n = (N + SK_BN - 1) / SK_BN;
-    int s = (256 + tiles_n / 2) / tiles_n;
+    int s = (192 + tiles_n / 2) / tiles_n;
     if (s < 1) s = 1;
     if (s > 16) s = 16;
     while (s > 1 && K / BK < 8 * s) --s;

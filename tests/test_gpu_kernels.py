@@ -352,10 +352,10 @@ def test_weight_streaming_gemm_small_shapes(ops, M, N, K):
     assert bool(((g - w_).abs() <= 2 ** -7 * w_.abs() + 2e-4 * w_.abs().max()).all())
 
 
-@pytest.mark.parametrize("M,N,K,split", [(128, 4096, 4096, 8), (100, 6144, 4096, 5), (128, 14336, 4096, 2),
-                                         (128, 4096, 14336, 8), (16, 1024, 1024, 2)])
+@pytest.mark.parametrize("M,N,K,split", [(128, 4096, 4096, 6), (100, 6144, 4096, 4), (128, 14336, 4096, 2),
+                                         (128, 4096, 14336, 6), (16, 1024, 1024, 2)])
 def test_weight_streaming_gemm_decode_shapes(ops, M, N, K, split):
-    """M <= 128: the plan picks the weight-streaming kernel and splits K so that about 256 workgroups stream W;
+    """M <= 128: the plan picks the weight-streaming kernel and splits K so that about 200 workgroups stream W;
     the parts are added in a fixed order, so the result is the same on every run."""
     import ctypes
 
