@@ -12,6 +12,15 @@
 // (qrow, half) are the probabilities of positions 8*half .. 8*half+7: exactly the lane's B fragment of
 // the first 16-position k-step of P V; registers 8..15 are the second.  Every accumulator of a lane
 // belongs to the lane's own query row, so the softmax statistics and the rescaling are lane-local.
+//
+// Two instantiations.  The fast one (SAFE = false) never rescales: every row keeps the maximum of its
+// first tile as the reference of its exponentials (mathematically the reference is arbitrary).  That
+// removes all arithmetic on the 128 output accumulators from the loop - they stay in the accumulation
+// registers from first to last tile.  Exponents can only overflow if a later score exceeds the row's first
+// maximum by more than 2^SAFE_LIMIT; a workgroup that sees this raises its flag in the workspace, and
+// the safe instantiation (running maximum, rescaling whenever the maximum moves by more than
+// 2^RESCALE_THRESHOLD), launched right behind on the same stream, recomputes exactly the flagged
+// workgroups and lowers the flags again.  Without flags it costs one load per workgroup.
 #include "dfhip_common.h"
 
 namespace {
@@ -25,6 +34,7 @@ constexpr int STAGE_BYTES = 2 * K_BYTES;         // K block + V block
 constexpr int ATT_LDS = STAGES * STAGE_BYTES;    // 96 KiB
 constexpr int OROW = AD * 2 + 16;                // padded row of the output staging area (bytes)
 constexpr float RESCALE_THRESHOLD = 8.0f;        // in units of log2: stale maxima up to 2^8 are tolerated
+constexpr float SAFE_LIMIT = 100.0f;             // fast path: scores may exceed the row's reference by 2^100
 
 DFHIP_DEVICE int pi(int m) {   // MFMA row -> position inside a 32-position tile
   const int g = (m >> 2) & 3;
@@ -32,10 +42,15 @@ DFHIP_DEVICE int pi(int m) {   // MFMA row -> position inside a 32-position tile
   return (m & 16) | (g2 << 2) | (m & 3);
 }
 
+template <bool SAFE>
 __global__ void __launch_bounds__(256)
 causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint16_t* __restrict__ k, int64_t ld_k,
                         const uint16_t* __restrict__ v_blk, uint16_t* __restrict__ out, int64_t ld_o, int B, int S,
-                        int q_heads, int kv_heads, float scale_log2) {
+                        int q_heads, int kv_heads, float scale_log2, int* __restrict__ flags) {
+  if (SAFE) {
+    if (flags[blockIdx.x] == 0) return;        // nothing to repair here (uniform over the workgroup)
+  }
+  bool risk = false;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -134,7 +149,9 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
     const bool diagonal = j == last_block_wave;
     const uint8_t* kst = smem + stage * STAGE_BYTES;
     const uint8_t* vst = kst + K_BYTES;
-#pragma unroll
+    // not unrolled: with two copies of the body in flight the register allocator starts moving the output
+    // accumulators between the accumulation and the vector registers inside the loop
+#pragma clang loop unroll(disable)
     for (int sb = 0; sb < 2; ++sb) {
       f32x16 s[2];
 #pragma unroll
@@ -164,16 +181,21 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
 #pragma unroll
         for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, s[nb][r]);
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        // keep a stale maximum while the scores stay within 2^RESCALE_THRESHOLD of it
-        if (__any((tmax - m_run[nb]) * scale_log2 > RESCALE_THRESHOLD)) {
-          const float m_new = fmaxf(m_run[nb], tmax);
-          const float alpha = __builtin_amdgcn_exp2f((m_run[nb] - m_new) * scale_log2);   // 0 on the first block
-          m_run[nb] = m_new;
-          l_run[nb] *= alpha;
+        if (SAFE) {
+          // keep a stale maximum while the scores stay within 2^RESCALE_THRESHOLD of it
+          if (__any((tmax - m_run[nb]) * scale_log2 > RESCALE_THRESHOLD)) {
+            const float m_new = fmaxf(m_run[nb], tmax);
+            const float alpha = __builtin_amdgcn_exp2f((m_run[nb] - m_new) * scale_log2);   // 0 on the first block
+            m_run[nb] = m_new;
+            l_run[nb] *= alpha;
 #pragma unroll
-          for (int db = 0; db < 4; ++db)
+            for (int db = 0; db < 4; ++db)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o[db][nb][r] *= alpha;
+              for (int r = 0; r < 16; ++r) o[db][nb][r] *= alpha;
+          }
+        } else {
+          if (m_run[nb] == -INFINITY) m_run[nb] = tmax;   // first tile of the row: its maximum is the reference
+          risk |= (tmax - m_run[nb]) * scale_log2 > SAFE_LIMIT;
         }
         const float mc = m_run[nb] * scale_log2;
         float lsum = 0.0f;
@@ -197,6 +219,11 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
   }
   wait_vmcnt<0>();        // the dead re-reads of the last iterations
   workgroup_barrier();    // every wave is done with the stages: they become the output staging area
+  if (SAFE) {
+    if (tid == 0) flags[blockIdx.x] = 0;
+  } else if (__any(risk) && lane == 0) {
+    flags[blockIdx.x] = 1;   // the output of this workgroup is recomputed by the safe instantiation
+  }
 
   uint8_t* park = smem + wave * (64 * OROW);
 #pragma unroll
@@ -256,29 +283,45 @@ extern "C" int dfhip_pack_v_bf16(const void* v, int64_t ld_v, void* v_blk, int B
   return dfhip_check_launch();
 }
 
+extern "C" size_t dfhip_causal_attention_workspace_bytes(int B, int S, int q_heads) {
+  if (B < 1 || S < 1 || q_heads < 1) return 0;
+  return (size_t)B * q_heads * ((S + QROWS - 1) / QROWS) * sizeof(int);
+}
+
 extern "C" int dfhip_causal_attention_bf16(const void* q, int64_t ld_q, const void* k, int64_t ld_k,
                                            const void* v_blk, void* out, int64_t ld_o, int B, int S, int q_heads,
-                                           int kv_heads, int head_dim, float scale, dfhip_stream_t stream) {
-  if (!q || !k || !v_blk || !out) return DFHIP_ERR_NULL_POINTER;
+                                           int kv_heads, int head_dim, float scale, void* workspace,
+                                           size_t workspace_bytes, dfhip_stream_t stream) {
+  if (!q || !k || !v_blk || !out || !workspace) return DFHIP_ERR_NULL_POINTER;
   if (B < 1 || S < KVB || S % KVB != 0 || q_heads < 1 || kv_heads < 1 || q_heads % kv_heads != 0 || head_dim != AD)
     return DFHIP_ERR_BAD_SHAPE;
   const int64_t groups = (int64_t)B * q_heads * ((S + QROWS - 1) / QROWS);
   if (groups >= (int64_t)1 << 31) return DFHIP_ERR_BAD_SHAPE;
+  if (workspace_bytes < dfhip_causal_attention_workspace_bytes(B, S, q_heads)) return DFHIP_ERR_BAD_ARGUMENT;
   if (ld_q < (int64_t)q_heads * AD || ld_k < (int64_t)kv_heads * AD || ld_o < (int64_t)q_heads * AD)
     return DFHIP_ERR_BAD_STRIDE;
   if (ld_q % 8 || ld_k % 8 || ld_o % 8 || !dfhip_aligned16(q) || !dfhip_aligned16(k) || !dfhip_aligned16(v_blk) ||
-      !dfhip_aligned16(out))
+      !dfhip_aligned16(out) || (reinterpret_cast<uintptr_t>(workspace) & 3u))
     return DFHIP_ERR_BAD_ALIGNMENT;
   static bool lds_opted_in = false;
   if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(causal_attention_kernel),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(causal_attention_kernel<false>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, ATT_LDS) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(causal_attention_kernel<true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, ATT_LDS) != hipSuccess)
       return DFHIP_ERR_LAUNCH;
     lds_opted_in = true;
   }
-  hipLaunchKernelGGL(causal_attention_kernel, dim3((unsigned)groups), dim3(256), ATT_LDS,
-                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(q), ld_q,
-                     static_cast<const uint16_t*>(k), ld_k, static_cast<const uint16_t*>(v_blk),
-                     static_cast<uint16_t*>(out), ld_o, B, S, q_heads, kv_heads, scale * 1.4426950408889634f);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const float scale_log2 = scale * 1.4426950408889634f;
+  hipLaunchKernelGGL(causal_attention_kernel<false>, dim3((unsigned)groups), dim3(256), ATT_LDS, s,
+                     static_cast<const uint16_t*>(q), ld_q, static_cast<const uint16_t*>(k), ld_k,
+                     static_cast<const uint16_t*>(v_blk), static_cast<uint16_t*>(out), ld_o, B, S, q_heads, kv_heads,
+                     scale_log2, static_cast<int*>(workspace));
+  if (int rc = dfhip_check_launch()) return rc;
+  hipLaunchKernelGGL(causal_attention_kernel<true>, dim3((unsigned)groups), dim3(256), ATT_LDS, s,
+                     static_cast<const uint16_t*>(q), ld_q, static_cast<const uint16_t*>(k), ld_k,
+                     static_cast<const uint16_t*>(v_blk), static_cast<uint16_t*>(out), ld_o, B, S, q_heads, kv_heads,
+                     scale_log2, static_cast<int*>(workspace));
   return dfhip_check_launch();
 }

@@ -82,25 +82,34 @@ def _require_device(*tensors: torch.Tensor) -> None:
 #: split-K workspaces, one per (device, stream): launches on one stream run one after the
 #: other, launches on different streams may overlap and must not share arrival counters
 _splitk_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+_attention_workspaces: dict[tuple[int, int], torch.Tensor] = {}
 #: split K for shapes with too few tiles (DYNAFLOW_SPLIT_K=0 switches it off)
 SPLIT_K_ENABLED = os.environ.get("DYNAFLOW_SPLIT_K", "1") != "0"
 
 
-def _splitk_workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
+def _zeroed_workspace(cache: dict, device: torch.device, stream: int, nbytes: int, clear: int = 65536) -> torch.Tensor:
+    """A per-(device, stream) scratch buffer whose first ``clear`` bytes are zero at first use.
+
+    The kernels that use these buffers (split-K arrival counters, attention repair flags) leave them zero.
+    """
     key = (device.index or 0, stream)
-    ws = _splitk_workspaces.get(key)
+    ws = cache.get(key)
     if torch.cuda.is_current_stream_capturing() and (ws is None or ws.numel() < nbytes):
-        # A capture on a stream of its own (per-sub-graph graphs): the workspace comes from the graph's
-        # memory pool and its counter area (at the start; 64 KiB are cleared) is zeroed by a fill kernel that is part of
-        # the graph - no memset node.  Graphs of one pool replay one after the other, so they may share.
+        # A capture on a stream of its own (per-sub-graph graphs): the buffer comes from the graph's
+        # memory pool and its start is zeroed by a fill kernel that is part of the graph - no memset
+        # node.  Graphs of one pool replay one after the other, so they may share.
         ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        rc = _cabi.load().dfhip_fill_u32(ws.data_ptr(), 0, min(nbytes, 65536) // 4, stream)
+        rc = _cabi.load().dfhip_fill_u32(ws.data_ptr(), 0, min(nbytes, clear) // 4, stream)
         _cabi.check("dfhip_fill_u32", rc)
         return ws
     if ws is None or ws.numel() < nbytes:
         ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
-        _splitk_workspaces[key] = ws
+        cache[key] = ws
     return ws
+
+
+def _splitk_workspace(device: torch.device, stream: int, nbytes: int) -> torch.Tensor:
+    return _zeroed_workspace(_splitk_workspaces, device, stream, nbytes)
 
 
 def _plan_bf16(lib, M: int, N: int, K: int) -> tuple[int, int]:
@@ -363,9 +372,11 @@ def _causal_attention_impl(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) ->
         stream = _stream()
         rc = lib.dfhip_pack_v_bf16(v.data_ptr(), ld_v, v_blk.data_ptr(), B, S, Hkv, d, stream)
         _cabi.check("dfhip_pack_v_bf16", rc)
+        nbytes = max(256, lib.dfhip_causal_attention_workspace_bytes(B, S, Hq))
+        flags = _zeroed_workspace(_attention_workspaces, q.device, stream, nbytes)
         rc = lib.dfhip_causal_attention_bf16(
             q.data_ptr(), ld_q, k.data_ptr(), ld_k, v_blk.data_ptr(), out.data_ptr(), Hq * d, B, S, Hq, Hkv, d,
-            1.0 / math.sqrt(d), stream,
+            1.0 / math.sqrt(d), flags.data_ptr(), flags.numel(), stream,
         )
         _cabi.check("dfhip_causal_attention_bf16", rc)
     return out

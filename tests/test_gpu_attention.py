@@ -102,3 +102,24 @@ def test_causal_attention_under_graph_capture(ops):
         torch.cuda.synchronize()
         assert torch.equal(out, eager), f"replay {i}"
         torch.randn(256, 256, device="cuda").sum().item()
+
+
+def test_causal_attention_scores_that_outgrow_the_first_tile(ops):
+    """Rows whose later scores exceed the maximum of their first tile by far more than 2^100: the fast launch
+    flags those workgroups and the repairing launch recomputes them with a running maximum.  Half of the
+    (sequence, head) pairs are affected, the others stay on the fast path; both must match the oracle, and the
+    flags must be lowered again (a second call gives the same bits)."""
+    B, S, Hq, Hkv = 2, 512, 4, 2
+    q, k, v = inputs(B, S, Hq, Hkv, 77)
+    direction = torch.nn.functional.normalize(torch.randn(D, generator=torch.Generator().manual_seed(1)), dim=0)
+    q[0] = (q[0].float() + 30.0 * direction).bfloat16()              # sequence 0: queries aligned with ...
+    k[0, 300:] = (k[0, 300:].float() + 30.0 * direction).bfloat16()  # ... the late keys: logits of about +80 nats
+    got = ops.causal_attention(q.cuda(), k.cuda(), v.cuda())
+    again = ops.causal_attention(q.cuda(), k.cuda(), v.cuda())
+    torch.cuda.synchronize()
+    want = ref.attention(q.double(), k.double(), v.double())
+    assert torch.isfinite(got.float()).all()
+    assert rel_err(got.float(), want) < TOL_BF16
+    err = (got.double().cpu() - want).abs().amax(dim=(2, 3))
+    assert bool((err < 0.05).all()), err.argmax()
+    assert torch.equal(got, again)
