@@ -58,6 +58,10 @@ def parse_args():
                    help="time the decode-step kernels at the shape of one nano-batch of the decode configuration "
                         "(128 sequences, 32 query / 8 kv heads, 2048 cached positions): RoPE + cache append + "
                         "attention, against the HBM roofline")
+    p.add_argument("--prefill-attention-kernels", action="store_true",
+                   help="time causal prefill attention at the shape of one nano-batch of the decoder-layer "
+                        "configuration (4 sequences x 2048 tokens, 32 query / 8 kv heads), PyTorch's fused "
+                        "attention beside it")
     p.add_argument("--decode", action="store_true",
                    help="measure one decode step over 32 stacked 8B-shaped layers (256 single-token queries, "
                         "2048 cached positions each, 2 nano-batches of 128) instead of the headline configuration")
@@ -168,6 +172,30 @@ def decode_kernels(torch, ops, iters):
         "roofline": {"kernel": "decode_attention_kernel", "bound": "hbm", "achieved": cache_bytes / (ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": cache_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "algorithmic_bytes": cache_bytes},
+    }
+
+
+def prefill_attention_kernels(torch, ops, iters):
+    """Causal grouped-query attention of one prefill nano-batch.  Algorithmic work: the causal half of the
+    two products, 2 * B * heads * S * S * d FLOP."""
+    B, S, heads, kv_heads, d = 4, 2048, 32, 8, 128
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    q = torch.randn(B, S, heads, d, generator=gen, device="cuda").bfloat16()
+    k = torch.randn(B, S, kv_heads, d, generator=gen, device="cuda").bfloat16()
+    v = torch.randn(B, S, kv_heads, d, generator=gen, device="cuda").bfloat16()
+    ms = time_kernel(torch, lambda: ops.causal_attention(q, k, v), iters)
+    qt, kt, vt = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
+    sdpa = torch.nn.functional.scaled_dot_product_attention
+    aten_ms = time_kernel(torch, lambda: sdpa(qt, kt, vt, is_causal=True, enable_gqa=True), iters)
+    flop = 2.0 * B * heads * S * S * d
+    return {
+        "workload": f"causal prefill attention, {B} sequences x {S} tokens, {heads} query / {kv_heads} kv heads, "
+                    f"head_dim {d}, bf16 (V re-layout kernel, attention kernel, repair pass)",
+        "ms": ms,
+        "torch_sdpa_ms": aten_ms,
+        "roofline": {"kernel": "causal_attention_fast_kernel", "bound": "mfma", "achieved": flop / (ms * 1e-3) / 1e12,
+                     "peak": BF16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flop / (ms * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, "algorithmic_flop": flop},
     }
 
 
@@ -432,6 +460,9 @@ def main() -> int:
         return 0
     if args.decode_kernels:
         print(json.dumps(decode_kernels(torch, ops, max(20, args.steps))))
+        return 0
+    if args.prefill_attention_kernels:
+        print(json.dumps(prefill_attention_kernels(torch, ops, max(20, args.steps))))
         return 0
     if args.fp8:
         print(json.dumps(fp8_config(torch, max(5, args.steps // 5), max(3, args.warmup // 5))))

@@ -13,14 +13,16 @@
 // the first 16-position k-step of P V; registers 8..15 are the second.  Every accumulator of a lane
 // belongs to the lane's own query row, so the softmax statistics and the rescaling are lane-local.
 //
-// Two instantiations.  The fast one (SAFE = false) never rescales: every row keeps the maximum of its
-// first tile as the reference of its exponentials (mathematically the reference is arbitrary).  That
-// removes all arithmetic on the 128 output accumulators from the loop - they stay in the accumulation
-// registers from first to last tile.  Exponents can only overflow if a later score exceeds the row's first
-// maximum by more than 2^SAFE_LIMIT; a workgroup that sees this raises its flag in the workspace, and
-// the safe instantiation (running maximum, rescaling whenever the maximum moves by more than
-// 2^RESCALE_THRESHOLD), launched right behind on the same stream, recomputes exactly the flagged
-// workgroups and lowers the flags again.  Without flags it costs one load per workgroup.
+// Two kernels.  The fast one never rescales: every row keeps the maximum of its first tile as the
+// reference of its exponentials (mathematically the reference is arbitrary).  That removes all arithmetic
+// on the 128 output accumulators from the loop - they stay in the accumulation registers from first to
+// last tile.  Exponents can only overflow if a later score exceeds the row's first maximum by more than
+// 2^SAFE_LIMIT; a workgroup that sees this raises its flag in the workspace, and the safe kernel (running
+// maximum, rescaling whenever the maximum moves by more than 2^RESCALE_THRESHOLD), launched right behind
+// on the same stream, recomputes exactly the flagged workgroups and lowers the flags again.  Without flags
+// it costs one load per workgroup.
+#include <type_traits>
+
 #include "dfhip_common.h"
 
 namespace {
@@ -36,33 +38,27 @@ constexpr int OROW = AD * 2 + 16;                // padded row of the output sta
 constexpr float RESCALE_THRESHOLD = 8.0f;        // in units of log2: stale maxima up to 2^8 are tolerated
 constexpr float SAFE_LIMIT = 100.0f;             // fast path: scores may exceed the row's reference by 2^100
 
+// maximum of three without the quieting of signalling NaNs that fmaxf implies (one instruction)
+DFHIP_DEVICE float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 DFHIP_DEVICE int pi(int m) {   // MFMA row -> position inside a 32-position tile
   const int g = (m >> 2) & 3;
   const int g2 = ((g & 1) << 1) | (g >> 1);      // 0,1,2,3 -> 0,2,1,3
   return (m & 16) | (g2 << 2) | (m & 3);
 }
 
-template <bool SAFE>
-__global__ void __launch_bounds__(256)
-causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint16_t* __restrict__ k, int64_t ld_k,
-                        const uint16_t* __restrict__ v_blk, uint16_t* __restrict__ out, int64_t ld_o, int B, int S,
-                        int q_heads, int kv_heads, float scale_log2, int* __restrict__ flags) {
-  if (SAFE) {
-    if (flags[blockIdx.x] == 0) return;        // nothing to repair here (uniform over the workgroup)
-  }
-  bool risk = false;
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int col = lane & 31, half = lane >> 5;
+// workgroup -> (sequence, kv head, query head, query block).  All query heads of a (sequence, kv head)
+// pair run on ONE XCD (its K and V stay in that XCD's L2); inside an XCD's range the heavy query blocks
+// (late rows, many K/V blocks) come first.
+DFHIP_DEVICE void map_workgroup(int B, int S, int q_heads, int kv_heads, int& b, int& kvh, int& hq, int& qb) {
   const int group = q_heads / kv_heads;
   const int nqb = (S + QROWS - 1) / QROWS;
-
-  // workgroup -> (sequence, kv head, head in group, query block).  All query heads of a (sequence, kv
-  // head) pair run on ONE XCD (its K and V stay in that XCD's L2); inside an XCD's range the heavy query
-  // blocks (late rows, many K/V blocks) come first.
   const int sets = B * kv_heads;
-  int b, kvh, hg, qb;
+  int hg;
   if (sets % 8 == 0) {
     const int total = sets * group * nqb;
     const int t = remap_xcd(blockIdx.x, total);
@@ -83,7 +79,54 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
     b = set / kv_heads;
     kvh = set % kv_heads;
   }
-  const int hq = kvh * group + hg;
+  hq = kvh * group + hg;
+}
+
+// O^T accumulators of a wave (64 query rows) -> out rows, through the wave's LDS staging area
+DFHIP_DEVICE void store_output(uint8_t* smem, const f32x16 (&o)[4][2], const float (&l_run)[2],
+                               uint16_t* __restrict__ out, int64_t ld_o, int b, int S, int hq, int q0, int wave,
+                               int lane) {
+  const int col = lane & 31, half = lane >> 5;
+  uint8_t* park = smem + wave * (64 * OROW);
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    const float l_tot = l_run[nb] + __shfl_xor(l_run[nb], 32, 64);
+    const float inv = 1.0f / l_tot;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w;
+        w[0] = pack2_bf16(o[db][nb][4 * g + 0] * inv, o[db][nb][4 * g + 1] * inv);
+        w[1] = pack2_bf16(o[db][nb][4 * g + 2] * inv, o[db][nb][4 * g + 3] * inv);
+        *reinterpret_cast<u32x2*>(park + (nb * 32 + col) * OROW + (db * 32 + 8 * g + 4 * half) * 2) = w;
+      }
+  }
+  DFHIP_PIN;
+  const int64_t row0 = (int64_t)b * S + q0 + wave * 64;
+#pragma unroll 4
+  for (int p = 0; p < 16; ++p) {
+    const int id = p * 64 + lane;
+    const int row = id >> 4, c = id & 15;
+    const u32x4 w = *reinterpret_cast<const u32x4*>(park + row * OROW + c * 16);
+    if (q0 + wave * 64 + row < S)
+      *reinterpret_cast<u32x4*>(out + (row0 + row) * ld_o + (int64_t)hq * AD + c * 8) = w;
+  }
+}
+
+// The safe kernel: running maximum, rescaling when it moves.  Recomputes the workgroups whose flag is up.
+__global__ void __launch_bounds__(256)
+causal_attention_safe_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint16_t* __restrict__ k,
+                             int64_t ld_k, const uint16_t* __restrict__ v_blk, uint16_t* __restrict__ out,
+                             int64_t ld_o, int B, int S, int q_heads, int kv_heads, float scale_log2,
+                             int* __restrict__ flags) {
+  if (flags[blockIdx.x] == 0) return;          // nothing to repair here (uniform over the workgroup)
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 31, half = lane >> 5;
+  int b, kvh, hq, qb;
+  map_workgroup(B, S, q_heads, kv_heads, b, kvh, hq, qb);
   const int q0 = qb * QROWS;                                  // first query row (inside the sequence)
   const int last_block_wg = ((q0 + QROWS < S ? q0 + QROWS : S) + KVB - 1) / KVB - 1;
   const int last_block_wave = q0 / KVB + wave;                 // the wave's diagonal block
@@ -181,21 +224,16 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
 #pragma unroll
         for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, s[nb][r]);
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        if (SAFE) {
-          // keep a stale maximum while the scores stay within 2^RESCALE_THRESHOLD of it
-          if (__any((tmax - m_run[nb]) * scale_log2 > RESCALE_THRESHOLD)) {
-            const float m_new = fmaxf(m_run[nb], tmax);
-            const float alpha = __builtin_amdgcn_exp2f((m_run[nb] - m_new) * scale_log2);   // 0 on the first block
-            m_run[nb] = m_new;
-            l_run[nb] *= alpha;
+        // keep a stale maximum while the scores stay within 2^RESCALE_THRESHOLD of it
+        if (__any((tmax - m_run[nb]) * scale_log2 > RESCALE_THRESHOLD)) {
+          const float m_new = fmaxf(m_run[nb], tmax);
+          const float alpha = __builtin_amdgcn_exp2f((m_run[nb] - m_new) * scale_log2);   // 0 on the first block
+          m_run[nb] = m_new;
+          l_run[nb] *= alpha;
 #pragma unroll
-            for (int db = 0; db < 4; ++db)
+          for (int db = 0; db < 4; ++db)
 #pragma unroll
-              for (int r = 0; r < 16; ++r) o[db][nb][r] *= alpha;
-          }
-        } else {
-          if (m_run[nb] == -INFINITY) m_run[nb] = tmax;   // first tile of the row: its maximum is the reference
-          risk |= (tmax - m_run[nb]) * scale_log2 > SAFE_LIMIT;
+            for (int r = 0; r < 16; ++r) o[db][nb][r] *= alpha;
         }
         const float mc = m_run[nb] * scale_log2;
         float lsum = 0.0f;
@@ -219,37 +257,249 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
   }
   wait_vmcnt<0>();        // the dead re-reads of the last iterations
   workgroup_barrier();    // every wave is done with the stages: they become the output staging area
-  if (SAFE) {
-    if (tid == 0) flags[blockIdx.x] = 0;
-  } else if (__any(risk) && lane == 0) {
-    flags[blockIdx.x] = 1;   // the output of this workgroup is recomputed by the safe instantiation
-  }
+  if (tid == 0) flags[blockIdx.x] = 0;
+  store_output(smem, o, l_run, out, ld_o, b, S, hq, q0, wave, lane);
+}
 
-  uint8_t* park = smem + wave * (64 * OROW);
+// The fast path, software-pipelined: with one wave per SIMD nothing else fills the matrix pipe while a
+// wave does its softmax, so every step of this kernel holds three independent pieces of work, interleaved
+// by hand and pinned - the P V MFMAs of tile t, the score MFMAs of tile t+2, and the softmax (VALU) of
+// tile t+1.  Score tiles and probability fragments alternate between two register sets (A: even tiles,
+// B: odd tiles).  K/V blocks live in a ring of 4 stages: block j (V in use), j+1 (K in use), j+2 and j+3
+// landing.  Rows keep the maximum of their first tile as reference (see above); flagged workgroups are
+// recomputed by the safe kernel.
+constexpr int FSTAGES = 4;
+constexpr int FATT_LDS = FSTAGES * STAGE_BYTES;  // 128 KiB
+
+__global__ void __launch_bounds__(256)
+causal_attention_fast_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint16_t* __restrict__ k,
+                             int64_t ld_k, const uint16_t* __restrict__ v_blk, uint16_t* __restrict__ out,
+                             int64_t ld_o, int B, int S, int q_heads, int kv_heads, float scale_log2,
+                             int* __restrict__ flags) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 31, half = lane >> 5;
+  int b, kvh, hq, qb;
+  map_workgroup(B, S, q_heads, kv_heads, b, kvh, hq, qb);
+  const int q0 = qb * QROWS;
+  const int last_block_wg = ((q0 + QROWS < S ? q0 + QROWS : S) + KVB - 1) / KVB - 1;
+  int last_block_wave = q0 / KVB + wave;                        // the wave's diagonal block
+  if (last_block_wave > last_block_wg) last_block_wave = last_block_wg;   // a wave of rows past S (never stored)
+
+  // ---- DMA sources: uniform bases that advance by one block, per-lane offsets fixed for the whole kernel
+  // (per block: 4 K instructions + 4 V instructions per wave, 1 KiB each)
+  const uint8_t* kseq = reinterpret_cast<const uint8_t*>(k + (int64_t)b * S * ld_k + (int64_t)kvh * AD);
+  const uint8_t* vseq = reinterpret_cast<const uint8_t*>(v_blk) + ((int64_t)(b * kv_heads + kvh) * S) * (AD * 2) +
+                        wave * 4096;
+  const int64_t k_block_bytes = (int64_t)KVB * ld_k * 2;
+  uint32_t k_off[4], v_off[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int row = (wave * 4 + t) * 4 + (lane >> 4);          // LDS row 0..63 (MFMA row order)
+    const int slot = lane & 15;
+    const int pos = (row & 32) | pi(row & 31);                 // position inside the block
+    const int chunk = (slot & 8) | ((slot & 7) ^ (row & 7));   // logical 16-byte chunk held by this slot
+    k_off[t] = (uint32_t)(pos * ld_k * 2 + chunk * 16);
+    v_off[t] = (uint32_t)(t * 1024 + lane * 16);
+  }
+  auto issue_block = [&](int j) {                               // nothing past the last block
+    if (j > last_block_wg) return;
+    const int stage = j % FSTAGES;
+    const uint8_t* kb = kseq + j * k_block_bytes;
+    const uint8_t* vb = vseq + (int64_t)j * (KVB * AD * 2);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) dma16_base(stage * STAGE_BYTES + (wave * 4 + t) * 1024, kb, k_off[t]);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) dma16_base(stage * STAGE_BYTES + K_BYTES + (wave * 4 + t) * 1024, vb, v_off[t]);
+  };
+
+  issue_block(0);
+  issue_block(1);
+  issue_block(2);
+  // ---- Q fragments (behind the first K/V blocks, so that everything is in flight together): B operand of
+  // S^T, lane supplies Q[qrow][16 ks + 8 half .. +8]
+  bf16x8 qf[2][8];
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-    const float l_tot = l_run[nb] + __shfl_xor(l_run[nb], 32, 64);
-    const float inv = 1.0f / l_tot;
+    int qrow = q0 + wave * 64 + nb * 32 + col;
+    qrow = qrow < S ? qrow : S - 1;
+    const uint16_t* qp = q + ((int64_t)b * S + qrow) * ld_q + (int64_t)hq * AD + 8 * half;
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int ks = 0; ks < 8; ++ks) qf[nb][ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
+  }
+
+
+  f32x16 o[4][2];
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w[0] = pack2_bf16(o[db][nb][4 * g + 0] * inv, o[db][nb][4 * g + 1] * inv);
-        w[1] = pack2_bf16(o[db][nb][4 * g + 2] * inv, o[db][nb][4 * g + 3] * inv);
-        *reinterpret_cast<u32x2*>(park + (nb * 32 + col) * OROW + (db * 32 + 8 * g + 4 * half) * 2) = w;
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[db][nb][r] = 0.0f;
+  float m_ref[2] = {0.0f, 0.0f};             // reference of the exponentials, already times scale_log2
+  float l_run[2] = {0.0f, 0.0f};
+  bool risk = false;
+  const int k_read = col * 256;
+  const int my_qrow0 = q0 + wave * 64 + col;
+
+  // LDS addresses of the A fragments: V pair p = (t, db) of tile [block, sb], K k-step ks of tile [block, sb]
+  auto v_frag = [&](int block, int sb, int p) {
+    const int t = p >> 2, db = p & 3;
+    return *reinterpret_cast<const bf16x8*>(smem + (block % FSTAGES) * STAGE_BYTES + K_BYTES +
+                                            ((sb * 4 + t * 2 + half) * AD + db * 32 + col) * 16);
+  };
+  auto k_frag = [&](int block, int sb, int ks) {
+    const int chunk = 2 * ks + half;
+    const int slot = (chunk & 8) | ((chunk & 7) ^ (col & 7));
+    return *reinterpret_cast<const bf16x8*>(smem + (block % FSTAGES) * STAGE_BYTES + sb * 8192 + k_read + slot * 16);
+  };
+
+  // The softmax of one score tile, cut into 26 slices (13 per half of the query rows) so that a slice can
+  // be placed behind every MFMA: 4 slices take the scores out of the accumulators and reduce 4 of them
+  // each, one fixes (FIRST) or checks the reference, 8 slices turn two scores each into probabilities.
+  float x[2][16], run_max[2], neg_ref[2] = {0.0f, 0.0f};
+  auto softmax_slice = [&](auto first, bool diag, int i, int block, int sb, const f32x16 (&s)[2],
+                           bf16x8 (&pf)[2][2]) {
+    const int nb = i / 13, c = i % 13;
+    if (c < 4) {
+      const int p_base = block * KVB + sb * 32 + 8 * half;
+      const int qrow = my_qrow0 + 32 * nb;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[nb][4 * c + e] = s[nb][4 * c + e];
+      if (diag) {                              // uniform over the wave
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = 4 * c + e;
+          if (p_base + 16 * (r >> 3) + (r & 7) > qrow) x[nb][r] = -INFINITY;
+        }
       }
+      if (c == 0) run_max[nb] = max3(x[nb][0], x[nb][1], max3(x[nb][0], x[nb][2], x[nb][3]));
+      else run_max[nb] = max3(max3(run_max[nb], x[nb][4 * c], x[nb][4 * c + 1]), x[nb][4 * c + 2], x[nb][4 * c + 3]);
+    } else if (c == 4) {
+      const float tmax = max3(run_max[nb], __shfl_xor(run_max[nb], 32, 64), run_max[nb]) * scale_log2;
+      if (decltype(first)::value) neg_ref[nb] = -tmax;       // first tile of the row: its maximum is the reference
+      else risk |= tmax + neg_ref[nb] > SAFE_LIMIT;
+    } else {
+      const int r = 2 * (c - 5);
+      const float p0 = __builtin_amdgcn_exp2f(fmaf(x[nb][r], scale_log2, neg_ref[nb]));
+      const float p1 = __builtin_amdgcn_exp2f(fmaf(x[nb][r + 1], scale_log2, neg_ref[nb]));
+      l_run[nb] += p0 + p1;
+      pf[nb][r >> 3][r & 7] = static_cast<bf16_t>(p0);
+      pf[nb][r >> 3][(r & 7) + 1] = static_cast<bf16_t>(p1);
+    }
+  };
+
+  // One step: P V of tile [vb, vsb] (probabilities pf_in), then - DO_S - the scores of tile [kb, ksb] into
+  // s_out, with - DO_SM - the softmax of tile [mb, msb] (scores s_in -> pf_out) sliced between the MFMAs.
+  // A fragments are read AHEAD MFMA pairs ahead; the first of a step are read by the step before (vpre),
+  // which is why the P V pairs come first: the V block of the next step has always landed already.
+  constexpr int AHEAD = 4;                     // pairs of MFMAs between a fragment's read and its use
+  bf16x8 vpre[AHEAD];
+  auto step = [&](auto do_s, auto do_sm, bool diag, int vb, int vsb, const bf16x8 (&pf_in)[2][2], int kb, int ksb,
+                  f32x16 (&s_out)[2], int mb, int msb, const f32x16 (&s_in)[2], bf16x8 (&pf_out)[2][2], int nvb,
+                  int nvsb) {
+    constexpr bool DO_S = decltype(do_s)::value, DO_SM = decltype(do_sm)::value;
+    constexpr int PAIRS = DO_S ? 16 : 8;
+    bf16x8 fr[PAIRS + AHEAD];
+#pragma unroll
+    for (int a = 0; a < AHEAD; ++a) fr[a] = vpre[a];
+#pragma unroll
+    for (int p = 0; p < PAIRS; ++p) {
+      const int n = p + AHEAD;                 // the fragment to fetch now
+      if (n < 8) fr[n] = v_frag(vb, vsb, n);
+      else if (n < PAIRS) fr[n] = k_frag(kb, ksb, n - 8);
+      else fr[n] = v_frag(nvb, nvsb, n - PAIRS);
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        if (p < 8) {
+          const int t = p >> 2, db = p & 3;
+          o[db][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[p], pf_in[nb][t], o[db][nb], 0, 0, 0);
+        } else if (p == 8) {
+          const f32x16 zero = {};
+          s_out[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[p], qf[nb][0], zero, 0, 0, 0);
+        } else {
+          s_out[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[p], qf[nb][p - 8], s_out[nb], 0, 0, 0);
+        }
+        if (DO_SM) {
+          const int m = 2 * p + nb;            // slices [26 m / (2 PAIRS), 26 (m+1) / (2 PAIRS))
+#pragma unroll
+          for (int i = 26 * m / (2 * PAIRS); i < 26 * (m + 1) / (2 * PAIRS); ++i)
+            softmax_slice(std::false_type{}, diag, i, mb, msb, s_in, pf_out);
+        }
+        DFHIP_PIN;
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < AHEAD; ++a) vpre[a] = fr[PAIRS + a];
+  };
+  using yes = std::true_type;
+  using no = std::false_type;
+
+  f32x16 sA[2], sB[2];
+  bf16x8 pfA[2][2], pfB[2][2];
+  wait_vmcnt<0>();                           // Q and the first blocks have landed
+  workgroup_barrier();
+  // prologue (not overlapped): scores of tiles 0 and 1, softmax of tile 0
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    f32x16 (&sd)[2] = t == 0 ? sA : sB;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const bf16x8 kf = k_frag(0, t, ks);
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        const f32x16 zero = {};
+        sd[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[nb][ks], ks == 0 ? zero : sd[nb], 0, 0, 0);
+      }
+    }
   }
-  DFHIP_PIN;
-  const int64_t row0 = (int64_t)b * S + q0 + wave * 64;
-#pragma unroll 4
-  for (int p = 0; p < 16; ++p) {
-    const int id = p * 64 + lane;
-    const int row = id >> 4, c = id & 15;
-    const u32x4 w = *reinterpret_cast<const u32x4*>(park + row * OROW + c * 16);
-    if (q0 + wave * 64 + row < S)
-      *reinterpret_cast<u32x4*>(out + (row0 + row) * ld_o + (int64_t)hq * AD + c * 8) = w;
+#pragma unroll
+  for (int i = 0; i < 26; ++i) softmax_slice(yes{}, last_block_wave == 0, i, 0, 0, sA, pfA);
+#pragma unroll
+  for (int a = 0; a < AHEAD; ++a) vpre[a] = v_frag(0, 0, a);
+
+  // Every wave passes last_block_wg + 1 barriers: full iterations up to its diagonal block, the drain of
+  // the diagonal block, then the staging duty only.  The three phases follow each other (no branch
+  // around code that touches the output accumulators, so they never leave the accumulation registers).
+  // Before iteration j block j+1 must have landed; only block j+2 (when there is one) may be in flight.
+  auto turn_ring = [&](int j) {
+    if (j + 2 <= last_block_wg) wait_vmcnt<8>();
+    else wait_vmcnt<0>();
+    workgroup_barrier();                     // block j+1 is there for every wave; everybody is done with block j-1
+    issue_block(j + 3);
+  };
+  int j = 0;
+  for (; j < last_block_wave; ++j) {
+    turn_ring(j);
+    step(yes{}, yes{}, false, j, 0, pfA, j + 1, 0, sA, j, 1, sB, pfB, j, 1);
+    step(yes{}, yes{}, j + 1 == last_block_wave, j, 1, pfB, j + 1, 1, sB, j + 1, 0, sA, pfA, j + 1, 0);
   }
+  turn_ring(j);
+  step(no{}, yes{}, true, j, 0, pfA, 0, 0, sA, j, 1, sB, pfB, j, 1);
+  step(no{}, no{}, false, j, 1, pfB, 0, 0, sA, 0, 0, sB, pfA, j, 1);
+  if (__any(risk) && lane == 0) flags[blockIdx.x] = 1;   // recomputed by the safe kernel
+
+  // The output goes from the registers straight to memory (a lane holds runs of 4 dims of its query rows), so
+  // a wave that is done stores while the others still work; its remaining duty is the ring.
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    const float inv = 1.0f / (l_run[nb] + __shfl_xor(l_run[nb], 32, 64));
+    const int qrow = q0 + wave * 64 + nb * 32 + col;
+    uint16_t* orow = out + ((int64_t)b * S + qrow) * ld_o + (int64_t)hq * AD + 4 * half;
+    if (qrow < S) {
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          u32x2 w;
+          w[0] = pack2_bf16(o[db][nb][4 * g + 0] * inv, o[db][nb][4 * g + 1] * inv);
+          w[1] = pack2_bf16(o[db][nb][4 * g + 2] * inv, o[db][nb][4 * g + 3] * inv);
+          *reinterpret_cast<u32x2*>(orow + db * 32 + 8 * g) = w;
+        }
+    }
+  }
+  for (++j; j <= last_block_wg; ++j) turn_ring(j);
 }
 
 // v[T, ld_v] (head h at column h*128) -> v_blk[B][kv_heads][S/8][128][8]
@@ -298,28 +548,29 @@ extern "C" int dfhip_causal_attention_bf16(const void* q, int64_t ld_q, const vo
   const int64_t groups = (int64_t)B * q_heads * ((S + QROWS - 1) / QROWS);
   if (groups >= (int64_t)1 << 31) return DFHIP_ERR_BAD_SHAPE;
   if (workspace_bytes < dfhip_causal_attention_workspace_bytes(B, S, q_heads)) return DFHIP_ERR_BAD_ARGUMENT;
-  if (ld_q < (int64_t)q_heads * AD || ld_k < (int64_t)kv_heads * AD || ld_o < (int64_t)q_heads * AD)
+  if (ld_q < (int64_t)q_heads * AD || ld_k < (int64_t)kv_heads * AD || ld_o < (int64_t)q_heads * AD ||
+      ld_k >= (int64_t)1 << 24)   // a K block's byte offsets are kept in 32 bits
     return DFHIP_ERR_BAD_STRIDE;
   if (ld_q % 8 || ld_k % 8 || ld_o % 8 || !dfhip_aligned16(q) || !dfhip_aligned16(k) || !dfhip_aligned16(v_blk) ||
       !dfhip_aligned16(out) || (reinterpret_cast<uintptr_t>(workspace) & 3u))
     return DFHIP_ERR_BAD_ALIGNMENT;
   static bool lds_opted_in = false;
   if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(causal_attention_kernel<false>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, ATT_LDS) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(causal_attention_kernel<true>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(causal_attention_fast_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, FATT_LDS) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(causal_attention_safe_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, ATT_LDS) != hipSuccess)
       return DFHIP_ERR_LAUNCH;
     lds_opted_in = true;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float scale_log2 = scale * 1.4426950408889634f;
-  hipLaunchKernelGGL(causal_attention_kernel<false>, dim3((unsigned)groups), dim3(256), ATT_LDS, s,
+  hipLaunchKernelGGL(causal_attention_fast_kernel, dim3((unsigned)groups), dim3(256), FATT_LDS, s,
                      static_cast<const uint16_t*>(q), ld_q, static_cast<const uint16_t*>(k), ld_k,
                      static_cast<const uint16_t*>(v_blk), static_cast<uint16_t*>(out), ld_o, B, S, q_heads, kv_heads,
                      scale_log2, static_cast<int*>(workspace));
   if (int rc = dfhip_check_launch()) return rc;
-  hipLaunchKernelGGL(causal_attention_kernel<true>, dim3((unsigned)groups), dim3(256), ATT_LDS, s,
+  hipLaunchKernelGGL(causal_attention_safe_kernel, dim3((unsigned)groups), dim3(256), ATT_LDS, s,
                      static_cast<const uint16_t*>(q), ld_q, static_cast<const uint16_t*>(k), ld_k,
                      static_cast<const uint16_t*>(v_blk), static_cast<uint16_t*>(out), ld_o, B, S, q_heads, kv_heads,
                      scale_log2, static_cast<int*>(workspace));

@@ -75,6 +75,11 @@ DFHIP_DEVICE void dma16(uint32_t lds_addr, const void* g) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(g)
                : "memory", "m0");
 }
+// The same with a wave-uniform base (scalar registers) and a 32-bit per-lane byte offset.
+DFHIP_DEVICE void dma16_base(uint32_t lds_addr, const void* base, uint32_t offset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(offset), "s"(base)
+               : "memory", "m0");
+}
 template <int N>
 DFHIP_DEVICE void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
