@@ -78,9 +78,8 @@ SIGNATURES: dict[str, tuple] = {
     "dfhip_rmsnorm_bf16": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, c_float, _P]),
     "dfhip_rope_bf16": (c_int, [_P, c_int64, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, _P]),
     "dfhip_pack_v_bf16": (c_int, [_P, c_int64, _P, c_int, c_int, c_int, c_int, _P]),
-    "dfhip_causal_attention_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "dfhip_causal_attention_bf16": (c_int, [_P, c_int64, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_int, c_int,
-                                            c_int, c_float, _P, c_size_t, _P]),
+                                            c_int, c_float, _P]),
     "dfhip_rope_kv_append_bf16": (c_int, [_P, c_int64, _P, c_int64, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
                                           c_int, c_int, c_int, _P]),
     "dfhip_decode_attention_bf16": (c_int, [_P, c_int64, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int,

@@ -13,14 +13,12 @@
 // the first 16-position k-step of P V; registers 8..15 are the second.  Every accumulator of a lane
 // belongs to the lane's own query row, so the softmax statistics and the rescaling are lane-local.
 //
-// Two kernels.  The fast one never rescales: every row keeps the maximum of its first tile as the
-// reference of its exponentials (mathematically the reference is arbitrary).  That removes all arithmetic
-// on the 128 output accumulators from the loop - they stay in the accumulation registers from first to
-// last tile.  Exponents can only overflow if a later score exceeds the row's first maximum by more than
-// 2^SAFE_LIMIT; a workgroup that sees this raises its flag in the workspace, and the safe kernel (running
-// maximum, rescaling whenever the maximum moves by more than 2^RESCALE_THRESHOLD), launched right behind
-// on the same stream, recomputes exactly the flagged workgroups and lowers the flags again.  Without flags
-// it costs one load per workgroup.
+// Two passes in one kernel.  The fast pass never rescales: every row keeps the maximum of its first tile
+// as the reference of its exponentials (mathematically the reference is arbitrary).  That removes all
+// arithmetic on the 128 output accumulators from the loop - they stay in the accumulation registers from
+// first to last tile.  Exponents can only overflow if a later score exceeds the row's first maximum by more
+// than 2^SAFE_LIMIT; a workgroup in which a wave sees this runs the safe pass behind the fast one (running
+// maximum, rescaling whenever the maximum moves by more than 2^RESCALE_THRESHOLD) and stores its rows again.
 #include <type_traits>
 
 #include "dfhip_common.h"
@@ -30,11 +28,10 @@ namespace {
 constexpr int AD = 128;          // head dim
 constexpr int QROWS = 256;       // query rows per workgroup
 constexpr int KVB = 64;          // positions per staged block
-constexpr int STAGES = 3;
+constexpr int STAGES = 4;
 constexpr int K_BYTES = KVB * AD * 2;            // 16 KiB
 constexpr int STAGE_BYTES = 2 * K_BYTES;         // K block + V block
-constexpr int ATT_LDS = STAGES * STAGE_BYTES;    // 96 KiB
-constexpr int OROW = AD * 2 + 16;                // padded row of the output staging area (bytes)
+constexpr int ATT_LDS = STAGES * STAGE_BYTES;    // 128 KiB
 constexpr float RESCALE_THRESHOLD = 8.0f;        // in units of log2: stale maxima up to 2^8 are tolerated
 constexpr float SAFE_LIMIT = 100.0f;             // fast path: scores may exceed the row's reference by 2^100
 
@@ -82,200 +79,15 @@ DFHIP_DEVICE void map_workgroup(int B, int S, int q_heads, int kv_heads, int& b,
   hq = kvh * group + hg;
 }
 
-// O^T accumulators of a wave (64 query rows) -> out rows, through the wave's LDS staging area
-DFHIP_DEVICE void store_output(uint8_t* smem, const f32x16 (&o)[4][2], const float (&l_run)[2],
-                               uint16_t* __restrict__ out, int64_t ld_o, int b, int S, int hq, int q0, int wave,
-                               int lane) {
-  const int col = lane & 31, half = lane >> 5;
-  uint8_t* park = smem + wave * (64 * OROW);
-#pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
-    const float l_tot = l_run[nb] + __shfl_xor(l_run[nb], 32, 64);
-    const float inv = 1.0f / l_tot;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w[0] = pack2_bf16(o[db][nb][4 * g + 0] * inv, o[db][nb][4 * g + 1] * inv);
-        w[1] = pack2_bf16(o[db][nb][4 * g + 2] * inv, o[db][nb][4 * g + 3] * inv);
-        *reinterpret_cast<u32x2*>(park + (nb * 32 + col) * OROW + (db * 32 + 8 * g + 4 * half) * 2) = w;
-      }
-  }
-  DFHIP_PIN;
-  const int64_t row0 = (int64_t)b * S + q0 + wave * 64;
-#pragma unroll 4
-  for (int p = 0; p < 16; ++p) {
-    const int id = p * 64 + lane;
-    const int row = id >> 4, c = id & 15;
-    const u32x4 w = *reinterpret_cast<const u32x4*>(park + row * OROW + c * 16);
-    if (q0 + wave * 64 + row < S)
-      *reinterpret_cast<u32x4*>(out + (row0 + row) * ld_o + (int64_t)hq * AD + c * 8) = w;
-  }
-}
-
-// The safe kernel: running maximum, rescaling when it moves.  Recomputes the workgroups whose flag is up.
+// The fast pass is software-pipelined: with one wave per SIMD nothing else fills the matrix pipe while a
+// wave does its softmax, so every step holds three independent pieces of work, interleaved by hand and
+// pinned - the P V MFMAs of tile t, the score MFMAs of tile t+2, and the softmax (VALU) of tile t+1.  Score
+// tiles and probability fragments alternate between two register sets (A: even tiles, B: odd tiles).  K/V
+// blocks live in a ring of 4 stages: block j (V in use), j+1 (K in use), j+2 and j+3 landing.
 __global__ void __launch_bounds__(256)
-causal_attention_safe_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint16_t* __restrict__ k,
-                             int64_t ld_k, const uint16_t* __restrict__ v_blk, uint16_t* __restrict__ out,
-                             int64_t ld_o, int B, int S, int q_heads, int kv_heads, float scale_log2,
-                             int* __restrict__ flags) {
-  if (flags[blockIdx.x] == 0) return;          // nothing to repair here (uniform over the workgroup)
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int col = lane & 31, half = lane >> 5;
-  int b, kvh, hq, qb;
-  map_workgroup(B, S, q_heads, kv_heads, b, kvh, hq, qb);
-  const int q0 = qb * QROWS;                                  // first query row (inside the sequence)
-  const int last_block_wg = ((q0 + QROWS < S ? q0 + QROWS : S) + KVB - 1) / KVB - 1;
-  const int last_block_wave = q0 / KVB + wave;                 // the wave's diagonal block
-
-  // ---- DMA sources (per block: 4 K instructions + 4 V instructions per wave, 1 KiB each)
-  const uint16_t* kseq = k + (int64_t)b * S * ld_k + (int64_t)kvh * AD;
-  const uint8_t* vseq = reinterpret_cast<const uint8_t*>(v_blk) + ((int64_t)(b * kv_heads + kvh) * S) * (AD * 2);
-  int k_row_off[4];      // position offset inside the block for LDS row (wave*4 + t)*4 + lane/16
-  int k_chunk[4];
-#pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int row = (wave * 4 + t) * 4 + (lane >> 4);          // LDS row 0..63 (MFMA row order)
-    const int slot = lane & 15;
-    k_row_off[t] = (row & 32) | pi(row & 31);
-    k_chunk[t] = (slot & 8) | ((slot & 7) ^ (row & 7));        // logical 16-byte chunk held by this slot
-  }
-  auto issue_block = [&](int j, int stage) {
-    const int jj = j <= last_block_wg ? j : last_block_wg;     // past the end: re-read into a dead stage
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      int pos = jj * KVB + k_row_off[t];
-      pos = pos < S ? pos : S - 1;
-      dma16(stage * STAGE_BYTES + (wave * 4 + t) * 1024, kseq + (int64_t)pos * ld_k + k_chunk[t] * 8);
-    }
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-      dma16(stage * STAGE_BYTES + K_BYTES + (wave * 4 + t) * 1024,
-            vseq + (int64_t)jj * (KVB * AD * 2) + (wave * 4 + t) * 1024 + lane * 16);
-  };
-
-  // ---- Q fragments: B operand of S^T, lane supplies Q[qrow][16 ks + 8 half .. +8]
-  bf16x8 qf[2][8];
-#pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
-    int qrow = q0 + wave * 64 + nb * 32 + col;
-    qrow = qrow < S ? qrow : S - 1;
-    const uint16_t* qp = q + ((int64_t)b * S + qrow) * ld_q + (int64_t)hq * AD + 8 * half;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[nb][ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
-  }
-
-  f32x16 o[4][2];
-#pragma unroll
-  for (int db = 0; db < 4; ++db)
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o[db][nb][r] = 0.0f;
-  float m_run[2] = {-INFINITY, -INFINITY};   // running (possibly stale) maximum of the raw scores
-  float l_run[2] = {0.0f, 0.0f};             // this lane's share of the row sum
-
-  issue_block(0, 0);
-  issue_block(1, 1);
-  const int k_read = col * 256;              // LDS row of this lane inside a 32-row tile
-  const int my_qrow0 = q0 + wave * 64 + col; // + 32 nb
-
-  for (int j = 0; j <= last_block_wg; ++j) {
-    const int stage = j % STAGES;
-    wait_vmcnt<8>();                         // block j has landed (block j+1 may be in flight)
-    workgroup_barrier();                     // ... for every wave; and everybody is done with block j-1
-    issue_block(j + 2, (j + 2) % STAGES);
-    if (j > last_block_wave) continue;       // beyond this wave's diagonal: only the staging duty
-    const bool diagonal = j == last_block_wave;
-    const uint8_t* kst = smem + stage * STAGE_BYTES;
-    const uint8_t* vst = kst + K_BYTES;
-    // not unrolled: with two copies of the body in flight the register allocator starts moving the output
-    // accumulators between the accumulation and the vector registers inside the loop
-#pragma clang loop unroll(disable)
-    for (int sb = 0; sb < 2; ++sb) {
-      f32x16 s[2];
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[nb][r] = 0.0f;
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const int chunk = 2 * ks + half;
-        const int slot = (chunk & 8) | ((chunk & 7) ^ (col & 7));
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kst + sb * 8192 + k_read + slot * 16);
-        s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[0][ks], s[0], 0, 0, 0);
-        s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[1][ks], s[1], 0, 0, 0);
-      }
-      // register r of this lane: position p_base + 16*(r/8) + (r%8), query row my_qrow0 + 32 nb
-      const int p_base = j * KVB + sb * 32 + 8 * half;
-      bf16x8 pf[2][2];
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb) {
-        if (diagonal) {
-          const int qrow = my_qrow0 + 32 * nb;
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            if (p_base + 16 * (r >> 3) + (r & 7) > qrow) s[nb][r] = -INFINITY;
-        }
-        float tmax = s[nb][0];
-#pragma unroll
-        for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, s[nb][r]);
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        // keep a stale maximum while the scores stay within 2^RESCALE_THRESHOLD of it
-        if (__any((tmax - m_run[nb]) * scale_log2 > RESCALE_THRESHOLD)) {
-          const float m_new = fmaxf(m_run[nb], tmax);
-          const float alpha = __builtin_amdgcn_exp2f((m_run[nb] - m_new) * scale_log2);   // 0 on the first block
-          m_run[nb] = m_new;
-          l_run[nb] *= alpha;
-#pragma unroll
-          for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o[db][nb][r] *= alpha;
-        }
-        const float mc = m_run[nb] * scale_log2;
-        float lsum = 0.0f;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float p = __builtin_amdgcn_exp2f(fmaf(s[nb][r], scale_log2, -mc));
-          lsum += p;
-          pf[nb][r >> 3][r & 7] = static_cast<bf16_t>(p);
-        }
-        l_run[nb] += lsum;
-      }
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vst + ((sb * 4 + t * 2 + half) * AD + db * 32 + col) * 16);
-          o[db][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[0][t], o[db][0], 0, 0, 0);
-          o[db][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[1][t], o[db][1], 0, 0, 0);
-        }
-    }
-  }
-  wait_vmcnt<0>();        // the dead re-reads of the last iterations
-  workgroup_barrier();    // every wave is done with the stages: they become the output staging area
-  if (tid == 0) flags[blockIdx.x] = 0;
-  store_output(smem, o, l_run, out, ld_o, b, S, hq, q0, wave, lane);
-}
-
-// The fast path, software-pipelined: with one wave per SIMD nothing else fills the matrix pipe while a
-// wave does its softmax, so every step of this kernel holds three independent pieces of work, interleaved
-// by hand and pinned - the P V MFMAs of tile t, the score MFMAs of tile t+2, and the softmax (VALU) of
-// tile t+1.  Score tiles and probability fragments alternate between two register sets (A: even tiles,
-// B: odd tiles).  K/V blocks live in a ring of 4 stages: block j (V in use), j+1 (K in use), j+2 and j+3
-// landing.  Rows keep the maximum of their first tile as reference (see above); flagged workgroups are
-// recomputed by the safe kernel.
-constexpr int FSTAGES = 4;
-constexpr int FATT_LDS = FSTAGES * STAGE_BYTES;  // 128 KiB
-
-__global__ void __launch_bounds__(256)
-causal_attention_fast_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint16_t* __restrict__ k,
-                             int64_t ld_k, const uint16_t* __restrict__ v_blk, uint16_t* __restrict__ out,
-                             int64_t ld_o, int B, int S, int q_heads, int kv_heads, float scale_log2,
-                             int* __restrict__ flags) {
+causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint16_t* __restrict__ k, int64_t ld_k,
+                        const uint16_t* __restrict__ v_blk, uint16_t* __restrict__ out, int64_t ld_o, int B, int S,
+                        int q_heads, int kv_heads, float scale_log2) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -305,7 +117,7 @@ causal_attention_fast_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const
   }
   auto issue_block = [&](int j) {                               // nothing past the last block
     if (j > last_block_wg) return;
-    const int stage = j % FSTAGES;
+    const int stage = j % STAGES;
     const uint8_t* kb = kseq + j * k_block_bytes;
     const uint8_t* vb = vseq + (int64_t)j * (KVB * AD * 2);
 #pragma unroll
@@ -337,7 +149,6 @@ causal_attention_fast_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const
     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[db][nb][r] = 0.0f;
-  float m_ref[2] = {0.0f, 0.0f};             // reference of the exponentials, already times scale_log2
   float l_run[2] = {0.0f, 0.0f};
   bool risk = false;
   const int k_read = col * 256;
@@ -346,13 +157,13 @@ causal_attention_fast_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const
   // LDS addresses of the A fragments: V pair p = (t, db) of tile [block, sb], K k-step ks of tile [block, sb]
   auto v_frag = [&](int block, int sb, int p) {
     const int t = p >> 2, db = p & 3;
-    return *reinterpret_cast<const bf16x8*>(smem + (block % FSTAGES) * STAGE_BYTES + K_BYTES +
+    return *reinterpret_cast<const bf16x8*>(smem + (block % STAGES) * STAGE_BYTES + K_BYTES +
                                             ((sb * 4 + t * 2 + half) * AD + db * 32 + col) * 16);
   };
   auto k_frag = [&](int block, int sb, int ks) {
     const int chunk = 2 * ks + half;
     const int slot = (chunk & 8) | ((chunk & 7) ^ (col & 7));
-    return *reinterpret_cast<const bf16x8*>(smem + (block % FSTAGES) * STAGE_BYTES + sb * 8192 + k_read + slot * 16);
+    return *reinterpret_cast<const bf16x8*>(smem + (block % STAGES) * STAGE_BYTES + sb * 8192 + k_read + slot * 16);
   };
 
   // The softmax of one score tile, cut into 26 slices (13 per half of the query rows) so that a slice can
@@ -478,28 +289,115 @@ causal_attention_fast_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const
   turn_ring(j);
   step(no{}, yes{}, true, j, 0, pfA, 0, 0, sA, j, 1, sB, pfB, j, 1);
   step(no{}, no{}, false, j, 1, pfB, 0, 0, sA, 0, 0, sB, pfA, j, 1);
-  if (__any(risk) && lane == 0) flags[blockIdx.x] = 1;   // recomputed by the safe kernel
-
   // The output goes from the registers straight to memory (a lane holds runs of 4 dims of its query rows), so
   // a wave that is done stores while the others still work; its remaining duty is the ring.
+  auto store_rows = [&]() {
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
-    const float inv = 1.0f / (l_run[nb] + __shfl_xor(l_run[nb], 32, 64));
-    const int qrow = q0 + wave * 64 + nb * 32 + col;
-    uint16_t* orow = out + ((int64_t)b * S + qrow) * ld_o + (int64_t)hq * AD + 4 * half;
-    if (qrow < S) {
+    for (int nb = 0; nb < 2; ++nb) {
+      const float inv = 1.0f / (l_run[nb] + __shfl_xor(l_run[nb], 32, 64));
+      const int qrow = q0 + wave * 64 + nb * 32 + col;
+      uint16_t* orow = out + ((int64_t)b * S + qrow) * ld_o + (int64_t)hq * AD + 4 * half;
+      if (qrow < S) {
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < 4; ++db)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          u32x2 w;
-          w[0] = pack2_bf16(o[db][nb][4 * g + 0] * inv, o[db][nb][4 * g + 1] * inv);
-          w[1] = pack2_bf16(o[db][nb][4 * g + 2] * inv, o[db][nb][4 * g + 3] * inv);
-          *reinterpret_cast<u32x2*>(orow + db * 32 + 8 * g) = w;
+          for (int g = 0; g < 4; ++g) {
+            u32x2 w;
+            w[0] = pack2_bf16(o[db][nb][4 * g + 0] * inv, o[db][nb][4 * g + 1] * inv);
+            w[1] = pack2_bf16(o[db][nb][4 * g + 2] * inv, o[db][nb][4 * g + 3] * inv);
+            *reinterpret_cast<u32x2*>(orow + db * 32 + 8 * g) = w;
+          }
+      }
+    }
+  };
+  store_rows();
+  for (++j; j <= last_block_wg; ++j) turn_ring(j);
+
+  // ---- Did any wave of the workgroup see a score beyond the reach of its reference?  (The ring is idle:
+  // the last turns waited for everything in flight.)
+  __syncthreads();
+  const bool wave_risk = __any(risk);
+  if (lane == 0) reinterpret_cast<int*>(smem)[wave] = wave_risk;
+  __syncthreads();
+  const int4 risks = *reinterpret_cast<const int4*>(smem);
+  if ((risks.x | risks.y | risks.z | risks.w) == 0) return;
+  __syncthreads();                           // everybody has read the four words before the ring restarts
+
+  // ---- The safe pass (rare): the whole workgroup again, tile by tile with a running maximum; the output
+  // accumulators are rescaled whenever the maximum moves by more than 2^RESCALE_THRESHOLD.  Same lanes, same
+  // addresses: the second store of a lane lands behind its first.
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[db][nb][r] = 0.0f;
+  float m_run[2] = {-INFINITY, -INFINITY};   // running (possibly stale) maximum of the raw scores
+  l_run[0] = l_run[1] = 0.0f;
+  issue_block(0);
+  for (int jb = 0; jb <= last_block_wg; ++jb) {
+    issue_block(jb + 1);                     // into a stage that neither block jb nor block jb-1 uses
+    if (jb + 1 <= last_block_wg) wait_vmcnt<8>();
+    else wait_vmcnt<0>();
+    workgroup_barrier();                     // block jb is there for every wave; everybody is done with jb-1
+    if (jb > last_block_wave) continue;
+    const bool diagonal = jb == last_block_wave;
+#pragma clang loop unroll(disable)
+    for (int sb = 0; sb < 2; ++sb) {
+      f32x16 s[2];
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const bf16x8 kf = k_frag(jb, sb, ks);
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+          const f32x16 zero = {};
+          s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[nb][ks], ks == 0 ? zero : s[nb], 0, 0, 0);
         }
+      }
+      // register r of this lane: position p_base + 16*(r/8) + (r%8), query row my_qrow0 + 32 nb
+      const int p_base = jb * KVB + sb * 32 + 8 * half;
+      bf16x8 pf[2][2];
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        if (diagonal) {
+          const int qrow = my_qrow0 + 32 * nb;
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (p_base + 16 * (r >> 3) + (r & 7) > qrow) s[nb][r] = -INFINITY;
+        }
+        float tmax = s[nb][0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, s[nb][r]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        if (__any((tmax - m_run[nb]) * scale_log2 > RESCALE_THRESHOLD)) {
+          const float m_new = fmaxf(m_run[nb], tmax);
+          const float alpha = __builtin_amdgcn_exp2f((m_run[nb] - m_new) * scale_log2);   // 0 on the first block
+          m_run[nb] = m_new;
+          l_run[nb] *= alpha;
+#pragma unroll
+          for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[db][nb][r] *= alpha;
+        }
+        const float mc = m_run[nb] * scale_log2;
+        float lsum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[nb][r], scale_log2, -mc));
+          lsum += p;
+          pf[nb][r >> 3][r & 7] = static_cast<bf16_t>(p);
+        }
+        l_run[nb] += lsum;
+      }
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        const bf16x8 vf = v_frag(jb, sb, p);
+        o[p & 3][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[0][p >> 2], o[p & 3][0], 0, 0, 0);
+        o[p & 3][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[1][p >> 2], o[p & 3][1], 0, 0, 0);
+      }
     }
   }
-  for (++j; j <= last_block_wg; ++j) turn_ring(j);
+  store_rows();
 }
 
 // v[T, ld_v] (head h at column h*128) -> v_blk[B][kv_heads][S/8][128][8]
@@ -533,46 +431,30 @@ extern "C" int dfhip_pack_v_bf16(const void* v, int64_t ld_v, void* v_blk, int B
   return dfhip_check_launch();
 }
 
-extern "C" size_t dfhip_causal_attention_workspace_bytes(int B, int S, int q_heads) {
-  if (B < 1 || S < 1 || q_heads < 1) return 0;
-  return (size_t)B * q_heads * ((S + QROWS - 1) / QROWS) * sizeof(int);
-}
-
 extern "C" int dfhip_causal_attention_bf16(const void* q, int64_t ld_q, const void* k, int64_t ld_k,
                                            const void* v_blk, void* out, int64_t ld_o, int B, int S, int q_heads,
-                                           int kv_heads, int head_dim, float scale, void* workspace,
-                                           size_t workspace_bytes, dfhip_stream_t stream) {
-  if (!q || !k || !v_blk || !out || !workspace) return DFHIP_ERR_NULL_POINTER;
+                                           int kv_heads, int head_dim, float scale, dfhip_stream_t stream) {
+  if (!q || !k || !v_blk || !out) return DFHIP_ERR_NULL_POINTER;
   if (B < 1 || S < KVB || S % KVB != 0 || q_heads < 1 || kv_heads < 1 || q_heads % kv_heads != 0 || head_dim != AD)
     return DFHIP_ERR_BAD_SHAPE;
   const int64_t groups = (int64_t)B * q_heads * ((S + QROWS - 1) / QROWS);
   if (groups >= (int64_t)1 << 31) return DFHIP_ERR_BAD_SHAPE;
-  if (workspace_bytes < dfhip_causal_attention_workspace_bytes(B, S, q_heads)) return DFHIP_ERR_BAD_ARGUMENT;
   if (ld_q < (int64_t)q_heads * AD || ld_k < (int64_t)kv_heads * AD || ld_o < (int64_t)q_heads * AD ||
       ld_k >= (int64_t)1 << 24)   // a K block's byte offsets are kept in 32 bits
     return DFHIP_ERR_BAD_STRIDE;
   if (ld_q % 8 || ld_k % 8 || ld_o % 8 || !dfhip_aligned16(q) || !dfhip_aligned16(k) || !dfhip_aligned16(v_blk) ||
-      !dfhip_aligned16(out) || (reinterpret_cast<uintptr_t>(workspace) & 3u))
+      !dfhip_aligned16(out))
     return DFHIP_ERR_BAD_ALIGNMENT;
   static bool lds_opted_in = false;
   if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(causal_attention_fast_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, FATT_LDS) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(causal_attention_safe_kernel),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(causal_attention_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, ATT_LDS) != hipSuccess)
       return DFHIP_ERR_LAUNCH;
     lds_opted_in = true;
   }
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const float scale_log2 = scale * 1.4426950408889634f;
-  hipLaunchKernelGGL(causal_attention_fast_kernel, dim3((unsigned)groups), dim3(256), FATT_LDS, s,
-                     static_cast<const uint16_t*>(q), ld_q, static_cast<const uint16_t*>(k), ld_k,
-                     static_cast<const uint16_t*>(v_blk), static_cast<uint16_t*>(out), ld_o, B, S, q_heads, kv_heads,
-                     scale_log2, static_cast<int*>(workspace));
-  if (int rc = dfhip_check_launch()) return rc;
-  hipLaunchKernelGGL(causal_attention_safe_kernel, dim3((unsigned)groups), dim3(256), ATT_LDS, s,
-                     static_cast<const uint16_t*>(q), ld_q, static_cast<const uint16_t*>(k), ld_k,
-                     static_cast<const uint16_t*>(v_blk), static_cast<uint16_t*>(out), ld_o, B, S, q_heads, kv_heads,
-                     scale_log2, static_cast<int*>(workspace));
+  hipLaunchKernelGGL(causal_attention_kernel, dim3((unsigned)groups), dim3(256), ATT_LDS,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(q), ld_q,
+                     static_cast<const uint16_t*>(k), ld_k, static_cast<const uint16_t*>(v_blk),
+                     static_cast<uint16_t*>(out), ld_o, B, S, q_heads, kv_heads, scale * 1.4426950408889634f);
   return dfhip_check_launch();
 }

@@ -82,7 +82,6 @@ def _require_device(*tensors: torch.Tensor) -> None:
 #: split-K workspaces, one per (device, stream): launches on one stream run one after the
 #: other, launches on different streams may overlap and must not share arrival counters
 _splitk_workspaces: dict[tuple[int, int], torch.Tensor] = {}
-_attention_workspaces: dict[tuple[int, int], torch.Tensor] = {}
 #: split K for shapes with too few tiles (DYNAFLOW_SPLIT_K=0 switches it off)
 SPLIT_K_ENABLED = os.environ.get("DYNAFLOW_SPLIT_K", "1") != "0"
 
@@ -90,7 +89,7 @@ SPLIT_K_ENABLED = os.environ.get("DYNAFLOW_SPLIT_K", "1") != "0"
 def _zeroed_workspace(cache: dict, device: torch.device, stream: int, nbytes: int, clear: int = 65536) -> torch.Tensor:
     """A per-(device, stream) scratch buffer whose first ``clear`` bytes are zero at first use.
 
-    The kernels that use these buffers (split-K arrival counters, attention repair flags) leave them zero.
+    The kernels that use these buffers (split-K arrival counters) leave them zero.
     """
     key = (device.index or 0, stream)
     ws = cache.get(key)
@@ -372,11 +371,9 @@ def _causal_attention_impl(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) ->
         stream = _stream()
         rc = lib.dfhip_pack_v_bf16(v.data_ptr(), ld_v, v_blk.data_ptr(), B, S, Hkv, d, stream)
         _cabi.check("dfhip_pack_v_bf16", rc)
-        nbytes = max(256, lib.dfhip_causal_attention_workspace_bytes(B, S, Hq))
-        flags = _zeroed_workspace(_attention_workspaces, q.device, stream, nbytes)
         rc = lib.dfhip_causal_attention_bf16(
             q.data_ptr(), ld_q, k.data_ptr(), ld_k, v_blk.data_ptr(), out.data_ptr(), Hq * d, B, S, Hq, Hkv, d,
-            1.0 / math.sqrt(d), flags.data_ptr(), flags.numel(), stream,
+            1.0 / math.sqrt(d), stream,
         )
         _cabi.check("dfhip_causal_attention_bf16", rc)
     return out

@@ -196,19 +196,17 @@ int dfhip_rope_bf16(const void* x, int64_t ld_x, void* out, int64_t ld_out, cons
  * fp32, probabilities rounded to bf16 for the second product, fp32 accumulation.
  * v is passed in the blocked layout v_blk[B][kv_heads][S/8][128][8] (8 consecutive
  * positions of one dim contiguous) that dfhip_pack_v_bf16 makes from v[B*S, ld_v].
- * workspace: one int per workgroup (dfhip_causal_attention_workspace_bytes),
- * ZERO before the first use and left zero: the first launch works without
- * rescaling its accumulators and flags the workgroups whose scores outgrow that
- * (by more than 2^100 over a row's first maximum), a second launch repairs those.
+ * One launch: a fast pass that never rescales its accumulators and, in the
+ * workgroups whose scores outgrow that (by more than 2^100 over a row's first
+ * maximum), a second pass with a running maximum.
  * In the reference this is the attention node of the host framework's model
  * graph (scaled_dot_product_attention of HF Llama, traced through
  * examples/ae/scripts/bench_hf_transformers.py:202-210); DynaFlow only schedules it. */
 int dfhip_pack_v_bf16(const void* v, int64_t ld_v, void* v_blk, int B, int S, int kv_heads, int head_dim,
                       dfhip_stream_t stream);
-size_t dfhip_causal_attention_workspace_bytes(int B, int S, int q_heads);
 int dfhip_causal_attention_bf16(const void* q, int64_t ld_q, const void* k, int64_t ld_k, const void* v_blk,
                                 void* out, int64_t ld_o, int B, int S, int q_heads, int kv_heads, int head_dim,
-                                float scale, void* workspace, size_t workspace_bytes, dfhip_stream_t stream);
+                                float scale, dfhip_stream_t stream);
 
 /* Decode step against a static KV cache (bf16, head_dim 128).  Cache layout, per
  * sequence slot and kv head, `capacity` positions (capacity % 32 == 0):
