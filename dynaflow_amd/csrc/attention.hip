@@ -16,9 +16,10 @@
 // Two passes in one kernel.  The fast pass never rescales: every row keeps the maximum of its first tile
 // as the reference of its exponentials (mathematically the reference is arbitrary).  That removes all
 // arithmetic on the 128 output accumulators from the loop - they stay in the accumulation registers from
-// first to last tile.  Exponents can only overflow if a later score exceeds the row's first maximum by more
-// than 2^SAFE_LIMIT; a workgroup in which a wave sees this runs the safe pass behind the fast one (running
-// maximum, rescaling whenever the maximum moves by more than 2^RESCALE_THRESHOLD) and stores its rows again.
+// first to last tile.  Exponentials and sums can only overflow if later scores exceed the row's first maximum
+// by far; a workgroup in which a row's sum of exponentials ends beyond SAFE_SUM runs the safe pass behind the
+// fast one (running maximum, rescaling whenever the maximum moves by more than 2^RESCALE_THRESHOLD) and
+// stores its rows again.
 #include <type_traits>
 
 #include "dfhip_common.h"
@@ -33,7 +34,7 @@ constexpr int K_BYTES = KVB * AD * 2;            // 16 KiB
 constexpr int STAGE_BYTES = 2 * K_BYTES;         // K block + V block
 constexpr int ATT_LDS = STAGES * STAGE_BYTES;    // 128 KiB
 constexpr float RESCALE_THRESHOLD = 8.0f;        // in units of log2: stale maxima up to 2^8 are tolerated
-constexpr float SAFE_LIMIT = 100.0f;             // fast path: scores may exceed the row's reference by 2^100
+constexpr float SAFE_SUM = 0x1p64f;               // fast pass: a row sum beyond this (relative to the row's reference) is redone
 
 // maximum of three without the quieting of signalling NaNs that fmaxf implies (one instruction)
 DFHIP_DEVICE float max3(float a, float b, float c) {
@@ -149,8 +150,6 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[db][nb][r] = 0.0f;
-  float l_run[2] = {0.0f, 0.0f};
-  bool risk = false;
   const int k_read = col * 256;
   const int my_qrow0 = q0 + wave * 64 + col;
 
@@ -166,83 +165,97 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
     return *reinterpret_cast<const bf16x8*>(smem + (block % STAGES) * STAGE_BYTES + sb * 8192 + k_read + slot * 16);
   };
 
-  // The softmax of one score tile, cut into 26 slices (13 per half of the query rows) so that a slice can
-  // be placed behind every MFMA: 4 slices take the scores out of the accumulators and reduce 4 of them
-  // each, one fixes (FIRST) or checks the reference, 8 slices turn two scores each into probabilities.
-  float x[2][16], run_max[2], neg_ref[2] = {0.0f, 0.0f};
-  auto softmax_slice = [&](auto first, bool diag, int i, int block, int sb, const f32x16 (&s)[2],
-                           bf16x8 (&pf)[2][2]) {
-    const int nb = i / 13, c = i % 13;
-    if (c < 4) {
-      const int p_base = block * KVB + sb * 32 + 8 * half;
+  // The reference of a row's exponentials (times scale_log2, negated): the maximum of its first tile.
+  float neg_ref[2] = {0.0f, 0.0f};
+  auto first_tile_reference = [&](bool diag, const f32x16 (&s)[2]) {
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
       const int qrow = my_qrow0 + 32 * nb;
+      float tmax = -INFINITY;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) x[nb][4 * c + e] = s[nb][4 * c + e];
-      if (diag) {                              // uniform over the wave
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = 4 * c + e;
-          if (p_base + 16 * (r >> 3) + (r & 7) > qrow) x[nb][r] = -INFINITY;
-        }
+      for (int r = 0; r < 16; ++r) {
+        const bool masked = diag && 8 * half + 16 * (r >> 3) + (r & 7) > qrow;   // tile 0 starts at position 0
+        tmax = fmaxf(tmax, masked ? -INFINITY : s[nb][r]);
       }
-      if (c == 0) run_max[nb] = max3(x[nb][0], x[nb][1], max3(x[nb][0], x[nb][2], x[nb][3]));
-      else run_max[nb] = max3(max3(run_max[nb], x[nb][4 * c], x[nb][4 * c + 1]), x[nb][4 * c + 2], x[nb][4 * c + 3]);
-    } else if (c == 4) {
-      const float tmax = max3(run_max[nb], __shfl_xor(run_max[nb], 32, 64), run_max[nb]) * scale_log2;
-      if (decltype(first)::value) neg_ref[nb] = -tmax;       // first tile of the row: its maximum is the reference
-      else risk |= tmax + neg_ref[nb] > SAFE_LIMIT;
-    } else {
-      const int r = 2 * (c - 5);
-      const float p0 = __builtin_amdgcn_exp2f(fmaf(x[nb][r], scale_log2, neg_ref[nb]));
-      const float p1 = __builtin_amdgcn_exp2f(fmaf(x[nb][r + 1], scale_log2, neg_ref[nb]));
-      l_run[nb] += p0 + p1;
-      pf[nb][r >> 3][r & 7] = static_cast<bf16_t>(p0);
-      pf[nb][r >> 3][(r & 7) + 1] = static_cast<bf16_t>(p1);
+      neg_ref[nb] = -fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * scale_log2;
     }
   };
+  // The softmax of one score tile in the fast pass is 16 slices (8 per half of the query rows), small enough
+  // to sit behind one MFMA each: a slice turns two scores into probabilities.  No maximum is taken and no
+  // sum: the row sums come out of the matrix pipe (an all-ones A operand against the probabilities), and
+  // whether a row's scores outgrew its reference shows in that sum at the end.
+  auto softmax_slice = [&](auto diag, int i, int block, int sb, const f32x16 (&s)[2], bf16x8 (&pf)[2][2]) {
+    const int nb = i >> 3, r = 2 * (i & 7);
+    float x0 = s[nb][r], x1 = s[nb][r + 1];
+    if (decltype(diag)::value) {
+      const int pos = block * KVB + sb * 32 + 8 * half + 16 * (r >> 3) + (r & 7);
+      const int qrow = my_qrow0 + 32 * nb;
+      if (pos > qrow) x0 = -INFINITY;
+      if (pos + 1 > qrow) x1 = -INFINITY;
+    }
+    pf[nb][r >> 3][r & 7] = static_cast<bf16_t>(__builtin_amdgcn_exp2f(fmaf(x0, scale_log2, neg_ref[nb])));
+    pf[nb][r >> 3][(r & 7) + 1] = static_cast<bf16_t>(__builtin_amdgcn_exp2f(fmaf(x1, scale_log2, neg_ref[nb])));
+  };
 
-  // One step: P V of tile [vb, vsb] (probabilities pf_in), then - DO_S - the scores of tile [kb, ksb] into
-  // s_out, with - DO_SM - the softmax of tile [mb, msb] (scores s_in -> pf_out) sliced between the MFMAs.
-  // A fragments are read AHEAD MFMA pairs ahead; the first of a step are read by the step before (vpre),
-  // which is why the P V pairs come first: the V block of the next step has always landed already.
-  constexpr int AHEAD = 4;                     // pairs of MFMAs between a fragment's read and its use
+  // One step: P V of tile [vb, vsb] (probabilities pf_in) with the two row-sum MFMAs of each k-step behind
+  // it, then - DO_S - the scores of tile [kb, ksb] into s_out, with - DO_SM - the softmax of tile [mb, msb]
+  // (scores s_in -> pf_out) sliced between the MFMAs.  A fragments are read AHEAD MFMA pairs ahead; the
+  // first of a step are read by the step before (vpre), which is why the P V pairs come first: the V block of
+  // the next step has always landed already.
+  constexpr int AHEAD = 4;                     // fragment-consuming pairs between a fragment's read and its use
   bf16x8 vpre[AHEAD];
-  auto step = [&](auto do_s, auto do_sm, bool diag, int vb, int vsb, const bf16x8 (&pf_in)[2][2], int kb, int ksb,
+  bf16x8 ones;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ones[e] = static_cast<bf16_t>(1.0f);
+  f32x16 l_acc[2];                             // every element: the row sum of the lane's query row
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) l_acc[nb][r] = 0.0f;
+  auto step = [&](auto do_s, auto do_sm, auto diag, int vb, int vsb, const bf16x8 (&pf_in)[2][2], int kb, int ksb,
                   f32x16 (&s_out)[2], int mb, int msb, const f32x16 (&s_in)[2], bf16x8 (&pf_out)[2][2], int nvb,
                   int nvsb) {
     constexpr bool DO_S = decltype(do_s)::value, DO_SM = decltype(do_sm)::value;
-    constexpr int PAIRS = DO_S ? 16 : 8;
-    bf16x8 fr[PAIRS + AHEAD];
+    constexpr int FRAGS = DO_S ? 16 : 8;       // pairs that consume an A fragment: 8 of P V, 8 of the scores
+    constexpr int PAIRS = FRAGS + 2;           // + the row sums of the two k-steps
+    bf16x8 fr[FRAGS + AHEAD];
 #pragma unroll
     for (int a = 0; a < AHEAD; ++a) fr[a] = vpre[a];
 #pragma unroll
-    for (int p = 0; p < PAIRS; ++p) {
-      const int n = p + AHEAD;                 // the fragment to fetch now
-      if (n < 8) fr[n] = v_frag(vb, vsb, n);
-      else if (n < PAIRS) fr[n] = k_frag(kb, ksb, n - 8);
-      else fr[n] = v_frag(nvb, nvsb, n - PAIRS);
+    for (int pq = 0; pq < PAIRS; ++pq) {
+      // pair order: pv0..pv3, sum(t=0), pv4..pv7, sum(t=1), score k-steps 0..7
+      const bool is_sum = pq == 4 || pq == 9;
+      const int f = pq < 4 ? pq : pq < 9 ? pq - 1 : pq - 2;      // fragment index of a consuming pair
+      if (!is_sum) {
+        const int n = f + AHEAD;               // the fragment to fetch now
+        if (n < 8) fr[n] = v_frag(vb, vsb, n);
+        else if (n < FRAGS) fr[n] = k_frag(kb, ksb, n - 8);
+        else fr[n] = v_frag(nvb, nvsb, n - FRAGS);
+      }
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb) {
-        if (p < 8) {
-          const int t = p >> 2, db = p & 3;
-          o[db][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[p], pf_in[nb][t], o[db][nb], 0, 0, 0);
-        } else if (p == 8) {
+        if (is_sum) {
+          l_acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pf_in[nb][pq == 4 ? 0 : 1], l_acc[nb], 0, 0, 0);
+        } else if (f < 8) {
+          const int t = f >> 2, db = f & 3;
+          o[db][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[f], pf_in[nb][t], o[db][nb], 0, 0, 0);
+        } else if (f == 8) {
           const f32x16 zero = {};
-          s_out[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[p], qf[nb][0], zero, 0, 0, 0);
+          s_out[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[f], qf[nb][0], zero, 0, 0, 0);
         } else {
-          s_out[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[p], qf[nb][p - 8], s_out[nb], 0, 0, 0);
+          s_out[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[f], qf[nb][f - 8], s_out[nb], 0, 0, 0);
         }
         if (DO_SM) {
-          const int m = 2 * p + nb;            // slices [26 m / (2 PAIRS), 26 (m+1) / (2 PAIRS))
+          const int m = 2 * pq + nb;           // slices [16 m / (2 PAIRS), 16 (m+1) / (2 PAIRS))
 #pragma unroll
-          for (int i = 26 * m / (2 * PAIRS); i < 26 * (m + 1) / (2 * PAIRS); ++i)
-            softmax_slice(std::false_type{}, diag, i, mb, msb, s_in, pf_out);
+          for (int i = 16 * m / (2 * PAIRS); i < 16 * (m + 1) / (2 * PAIRS); ++i)
+            softmax_slice(diag, i, mb, msb, s_in, pf_out);
         }
         DFHIP_PIN;
       }
     }
 #pragma unroll
-    for (int a = 0; a < AHEAD; ++a) vpre[a] = fr[PAIRS + a];
+    for (int a = 0; a < AHEAD; ++a) vpre[a] = fr[FRAGS + a];
   };
   using yes = std::true_type;
   using no = std::false_type;
@@ -265,8 +278,14 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
       }
     }
   }
+  first_tile_reference(last_block_wave == 0, sA);
+  if (last_block_wave == 0) {
 #pragma unroll
-  for (int i = 0; i < 26; ++i) softmax_slice(yes{}, last_block_wave == 0, i, 0, 0, sA, pfA);
+    for (int i = 0; i < 16; ++i) softmax_slice(yes{}, i, 0, 0, sA, pfA);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) softmax_slice(no{}, i, 0, 0, sA, pfA);
+  }
 #pragma unroll
   for (int a = 0; a < AHEAD; ++a) vpre[a] = v_frag(0, 0, a);
 
@@ -281,20 +300,26 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
     issue_block(j + 3);
   };
   int j = 0;
-  for (; j < last_block_wave; ++j) {
+  for (; j + 1 < last_block_wave; ++j) {
     turn_ring(j);
-    step(yes{}, yes{}, false, j, 0, pfA, j + 1, 0, sA, j, 1, sB, pfB, j, 1);
-    step(yes{}, yes{}, j + 1 == last_block_wave, j, 1, pfB, j + 1, 1, sB, j + 1, 0, sA, pfA, j + 1, 0);
+    step(yes{}, yes{}, no{}, j, 0, pfA, j + 1, 0, sA, j, 1, sB, pfB, j, 1);
+    step(yes{}, yes{}, no{}, j, 1, pfB, j + 1, 1, sB, j + 1, 0, sA, pfA, j + 1, 0);
+  }
+  if (j < last_block_wave) {                 // the block before the diagonal one: its second softmax is masked
+    turn_ring(j);
+    step(yes{}, yes{}, no{}, j, 0, pfA, j + 1, 0, sA, j, 1, sB, pfB, j, 1);
+    step(yes{}, yes{}, yes{}, j, 1, pfB, j + 1, 1, sB, j + 1, 0, sA, pfA, j + 1, 0);
+    ++j;
   }
   turn_ring(j);
-  step(no{}, yes{}, true, j, 0, pfA, 0, 0, sA, j, 1, sB, pfB, j, 1);
-  step(no{}, no{}, false, j, 1, pfB, 0, 0, sA, 0, 0, sB, pfA, j, 1);
+  step(no{}, yes{}, yes{}, j, 0, pfA, 0, 0, sA, j, 1, sB, pfB, j, 1);
+  step(no{}, no{}, no{}, j, 1, pfB, 0, 0, sA, 0, 0, sB, pfA, j, 1);
   // The output goes from the registers straight to memory (a lane holds runs of 4 dims of its query rows), so
   // a wave that is done stores while the others still work; its remaining duty is the ring.
-  auto store_rows = [&]() {
+  auto store_rows = [&](const float (&row_sum)[2]) {
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
-      const float inv = 1.0f / (l_run[nb] + __shfl_xor(l_run[nb], 32, 64));
+      const float inv = 1.0f / row_sum[nb];
       const int qrow = q0 + wave * 64 + nb * 32 + col;
       uint16_t* orow = out + ((int64_t)b * S + qrow) * ld_o + (int64_t)hq * AD + 4 * half;
       if (qrow < S) {
@@ -310,13 +335,14 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
       }
     }
   };
-  store_rows();
+  const float fast_sum[2] = {l_acc[0][0], l_acc[1][0]};
+  store_rows(fast_sum);
   for (++j; j <= last_block_wg; ++j) turn_ring(j);
 
-  // ---- Did any wave of the workgroup see a score beyond the reach of its reference?  (The ring is idle:
-  // the last turns waited for everything in flight.)
+  // ---- Did the scores of any row of the workgroup outgrow the row's reference?  Then exponentials or sums
+  // may have overflowed.  (The ring is idle: the last turns waited for everything in flight.)
   __syncthreads();
-  const bool wave_risk = __any(risk);
+  const bool wave_risk = __any(fast_sum[0] > SAFE_SUM || fast_sum[1] > SAFE_SUM);
   if (lane == 0) reinterpret_cast<int*>(smem)[wave] = wave_risk;
   __syncthreads();
   const int4 risks = *reinterpret_cast<const int4*>(smem);
@@ -333,7 +359,7 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[db][nb][r] = 0.0f;
   float m_run[2] = {-INFINITY, -INFINITY};   // running (possibly stale) maximum of the raw scores
-  l_run[0] = l_run[1] = 0.0f;
+  float l_run[2] = {0.0f, 0.0f};             // this lane's share of the row sum
   issue_block(0);
   for (int jb = 0; jb <= last_block_wg; ++jb) {
     issue_block(jb + 1);                     // into a stage that neither block jb nor block jb-1 uses
@@ -397,7 +423,8 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
       }
     }
   }
-  store_rows();
+  const float safe_sum[2] = {l_run[0] + __shfl_xor(l_run[0], 32, 64), l_run[1] + __shfl_xor(l_run[1], 32, 64)};
+  store_rows(safe_sum);
 }
 
 // v[T, ld_v] (head h at column h*128) -> v_blk[B][kv_heads][S/8][128][8]

@@ -196,9 +196,9 @@ int dfhip_rope_bf16(const void* x, int64_t ld_x, void* out, int64_t ld_out, cons
  * fp32, probabilities rounded to bf16 for the second product, fp32 accumulation.
  * v is passed in the blocked layout v_blk[B][kv_heads][S/8][128][8] (8 consecutive
  * positions of one dim contiguous) that dfhip_pack_v_bf16 makes from v[B*S, ld_v].
- * One launch: a fast pass that never rescales its accumulators and, in the
- * workgroups whose scores outgrow that (by more than 2^100 over a row's first
- * maximum), a second pass with a running maximum.
+ * One launch: a fast pass that never rescales its accumulators (a row's first
+ * tile fixes the reference of its exponentials) and, in the workgroups where a
+ * row's sum of exponentials ends beyond 2^64, a second pass with a running maximum.
  * In the reference this is the attention node of the host framework's model
  * graph (scaled_dot_product_attention of HF Llama, traced through
  * examples/ae/scripts/bench_hf_transformers.py:202-210); DynaFlow only schedules it. */

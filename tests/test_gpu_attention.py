@@ -105,10 +105,10 @@ def test_causal_attention_under_graph_capture(ops):
 
 
 def test_causal_attention_scores_that_outgrow_the_first_tile(ops):
-    """Rows whose later scores exceed the maximum of their first tile by far more than 2^100: the fast launch
-    flags those workgroups and the repairing launch recomputes them with a running maximum.  Half of the
-    (sequence, head) pairs are affected, the others stay on the fast path; both must match the oracle, and the
-    flags must be lowered again (a second call gives the same bits)."""
+    """Rows whose later scores exceed the maximum of their first tile by far more than 2^64: the fast pass
+    of those workgroups overflows its sums, notices, and the safe pass recomputes them with a running maximum.
+    Half of the (sequence, head) pairs are affected, the others stay on the fast pass; both must match the
+    oracle, and a second call gives the same bits."""
     B, S, Hq, Hkv = 2, 512, 4, 2
     q, k, v = inputs(B, S, Hq, Hkv, 77)
     direction = torch.nn.functional.normalize(torch.randn(D, generator=torch.Generator().manual_seed(1)), dim=0)
