@@ -116,15 +116,17 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
     k_off[t] = (uint32_t)(pos * ld_k * 2 + chunk * 16);
     v_off[t] = (uint32_t)(t * 1024 + lane * 16);
   }
-  auto issue_block = [&](int j) {                               // nothing past the last block
+  // piece t of block j: 4 K instructions (t = 0..3), then 4 V instructions; nothing past the last block
+  auto issue_piece = [&](int j, int t) {
     if (j > last_block_wg) return;
     const int stage = j % STAGES;
-    const uint8_t* kb = kseq + j * k_block_bytes;
-    const uint8_t* vb = vseq + (int64_t)j * (KVB * AD * 2);
+    if (t < 4) dma16_base(stage * STAGE_BYTES + (wave * 4 + t) * 1024, kseq + j * k_block_bytes, k_off[t]);
+    else dma16_base(stage * STAGE_BYTES + K_BYTES + (wave * 4 + t - 4) * 1024, vseq + (int64_t)j * (KVB * AD * 2),
+                    v_off[t - 4]);
+  };
+  auto issue_block = [&](int j) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t) dma16_base(stage * STAGE_BYTES + (wave * 4 + t) * 1024, kb, k_off[t]);
-#pragma unroll
-    for (int t = 0; t < 4; ++t) dma16_base(stage * STAGE_BYTES + K_BYTES + (wave * 4 + t) * 1024, vb, v_off[t]);
+    for (int t = 0; t < 8; ++t) issue_piece(j, t);
   };
 
   issue_block(0);
@@ -214,7 +216,7 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
     for (int r = 0; r < 16; ++r) l_acc[nb][r] = 0.0f;
   auto step = [&](auto do_s, auto do_sm, auto diag, int vb, int vsb, const bf16x8 (&pf_in)[2][2], int kb, int ksb,
                   f32x16 (&s_out)[2], int mb, int msb, const f32x16 (&s_in)[2], bf16x8 (&pf_out)[2][2], int nvb,
-                  int nvsb) {
+                  int nvsb, int dma_block) {
     constexpr bool DO_S = decltype(do_s)::value, DO_SM = decltype(do_sm)::value;
     constexpr int FRAGS = DO_S ? 16 : 8;       // pairs that consume an A fragment: 8 of P V, 8 of the scores
     constexpr int PAIRS = FRAGS + 2;           // + the row sums of the two k-steps
@@ -226,6 +228,11 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
       // pair order: pv0..pv3, sum(t=0), pv4..pv7, sum(t=1), score k-steps 0..7
       const bool is_sum = pq == 4 || pq == 9;
       const int f = pq < 4 ? pq : pq < 9 ? pq - 1 : pq - 2;      // fragment index of a consuming pair
+      // the 8 LDS-DMA instructions of the block that enters the ring in this iteration, spread over the step
+      // (4 waves issuing them in one burst keep the address unit, and with it the waves, busy for ~500 cycles)
+      if (dma_block >= 0) {
+        if (DO_S ? (pq & 1) && pq < 16 : pq < 8) issue_piece(dma_block, DO_S ? pq >> 1 : pq);
+      }
       if (!is_sum) {
         const int n = f + AHEAD;               // the fragment to fetch now
         if (n < 8) fr[n] = v_frag(vb, vsb, n);
@@ -257,6 +264,7 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
 #pragma unroll
     for (int a = 0; a < AHEAD; ++a) vpre[a] = fr[FRAGS + a];
   };
+  constexpr int NO_DMA = -1;
   using yes = std::true_type;
   using no = std::false_type;
 
@@ -297,23 +305,22 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
     if (j + 2 <= last_block_wg) wait_vmcnt<8>();
     else wait_vmcnt<0>();
     workgroup_barrier();                     // block j+1 is there for every wave; everybody is done with block j-1
-    issue_block(j + 3);
-  };
+  };                                         // ... so block j+3 may enter the ring (first step of the iteration)
   int j = 0;
   for (; j + 1 < last_block_wave; ++j) {
     turn_ring(j);
-    step(yes{}, yes{}, no{}, j, 0, pfA, j + 1, 0, sA, j, 1, sB, pfB, j, 1);
-    step(yes{}, yes{}, no{}, j, 1, pfB, j + 1, 1, sB, j + 1, 0, sA, pfA, j + 1, 0);
+    step(yes{}, yes{}, no{}, j, 0, pfA, j + 1, 0, sA, j, 1, sB, pfB, j, 1, j + 3);
+    step(yes{}, yes{}, no{}, j, 1, pfB, j + 1, 1, sB, j + 1, 0, sA, pfA, j + 1, 0, NO_DMA);
   }
   if (j < last_block_wave) {                 // the block before the diagonal one: its second softmax is masked
     turn_ring(j);
-    step(yes{}, yes{}, no{}, j, 0, pfA, j + 1, 0, sA, j, 1, sB, pfB, j, 1);
-    step(yes{}, yes{}, yes{}, j, 1, pfB, j + 1, 1, sB, j + 1, 0, sA, pfA, j + 1, 0);
+    step(yes{}, yes{}, no{}, j, 0, pfA, j + 1, 0, sA, j, 1, sB, pfB, j, 1, j + 3);
+    step(yes{}, yes{}, yes{}, j, 1, pfB, j + 1, 1, sB, j + 1, 0, sA, pfA, j + 1, 0, NO_DMA);
     ++j;
   }
   turn_ring(j);
-  step(no{}, yes{}, yes{}, j, 0, pfA, 0, 0, sA, j, 1, sB, pfB, j, 1);
-  step(no{}, no{}, no{}, j, 1, pfB, 0, 0, sA, 0, 0, sB, pfA, j, 1);
+  step(no{}, yes{}, yes{}, j, 0, pfA, 0, 0, sA, j, 1, sB, pfB, j, 1, j + 3);
+  step(no{}, no{}, no{}, j, 1, pfB, 0, 0, sA, 0, 0, sB, pfA, j, 1, NO_DMA);
   // The output goes from the registers straight to memory (a lane holds runs of 4 dims of its query rows), so
   // a wave that is done stores while the others still work; its remaining duty is the ring.
   auto store_rows = [&](const float (&row_sum)[2]) {
@@ -337,7 +344,10 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
   };
   const float fast_sum[2] = {l_acc[0][0], l_acc[1][0]};
   store_rows(fast_sum);
-  for (++j; j <= last_block_wg; ++j) turn_ring(j);
+  for (++j; j <= last_block_wg; ++j) {
+    turn_ring(j);
+    issue_block(j + 3);
+  }
 
   // ---- Did the scores of any row of the workgroup outgrow the row's reference?  Then exponentials or sums
   // may have overflowed.  (The ring is idle: the last turns waited for everything in flight.)
