@@ -14,6 +14,9 @@ it deep-copies the sub-``GraphModule`` and replaces
 * ``add(r, linear(x, w))`` (bf16, same shapes, the linear used once) -> ``dynaflow_hip.linear_add``
   (the residual addition as the GEMM's epilogue; same roundings, same bits)
 
+* the ``linear`` / ``linear_add`` whose result is what the sub-graph returns -> ``*_to_output``
+  (writes into rows offered by the engine, so the nano-batch outputs need no concatenation)
+
 With ``fuse_silu_epilogue`` a third rewrite follows: a ``silu_mul`` whose gate and up
 inputs are two bf16 ``linear`` nodes of the same activation becomes one
 ``dynaflow_hip.gate_up_silu(x, w_gate, w_up)`` - the SiLU*mul as the GEMM's epilogue.
@@ -273,6 +276,16 @@ def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False) -> tuple[
             stats["gate_up_silu"] += 1
             stats["linear"] -= 2
             stats["silu_mul"] -= 1
+
+    # The projection whose result the sub-graph returns (and nothing else reads) may write straight into the
+    # rows that the engine offers for the model output; without an offer it behaves like the plain operator.
+    output = next(n for n in graph.nodes if n.op == "output")
+    returned = output.args[0]
+    if isinstance(returned, fx.Node) and returned.op == "call_function" and len(returned.users) == 1:
+        into = {ops.linear: ops.linear_to_output, ops.linear_add: ops.linear_add_to_output}.get(returned.target)
+        if into is not None and not returned.kwargs:
+            returned.target = into
+            stats["to_output"] = 1
 
     graph.lint()
     lowered.recompile()

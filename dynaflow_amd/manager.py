@@ -58,15 +58,36 @@ def trivial_split(batch_size: int, num_tokens: list[int], is_dryrun: bool, use_c
     )
 
 
-def join_results(results: dict[int, Any], num_nano_batches: int) -> Any:
-    """Concatenate per-nano-batch outputs on dim 0 (tuples field by field)."""
+def _already_joined(parts: list[torch.Tensor], shared_buffer: torch.Tensor | None) -> torch.Tensor | None:
+    """The concatenation of ``parts`` on dim 0 without a copy, if they are consecutive row ranges that together
+    make up the engine's shared output buffer; else ``None``."""
+    base = parts[0]._base
+    if shared_buffer is None or base is not shared_buffer or not base.is_contiguous():
+        return None
+    offset, tail = base.storage_offset(), tuple(parts[0].shape[1:])
+    for part in parts:
+        if part._base is not base or not part.is_contiguous() or tuple(part.shape[1:]) != tail:
+            return None
+        if part.storage_offset() != offset:
+            return None
+        offset += part.numel()
+    if offset - base.storage_offset() != base.numel():
+        return None
+    rows = sum(part.shape[0] for part in parts)
+    return base.view(rows, *tail)
+
+
+def join_results(results: dict[int, Any], num_nano_batches: int, shared_buffer: torch.Tensor | None = None) -> Any:
+    """Concatenate per-nano-batch outputs on dim 0 (tuples field by field); outputs that already are the
+    consecutive rows of the engine's shared output buffer are returned as that buffer."""
     first = results[0]
     assert all(isinstance(r, type(first)) for r in results.values()), (
         f"Results have different types: {results}"
     )
     ordered = [results[b] for b in range(num_nano_batches)]
     if isinstance(first, torch.Tensor):
-        return torch.cat(ordered, dim=0)
+        joined = _already_joined(ordered, shared_buffer)
+        return joined if joined is not None else torch.cat(ordered, dim=0)
     if isinstance(first, tuple):
         width = len(first)
         assert all(len(r) == width for r in ordered), (
@@ -76,7 +97,8 @@ def join_results(results: dict[int, Any], num_nano_batches: int) -> Any:
         for i in range(width):
             column = [r[i] for r in ordered]
             assert all(isinstance(e, torch.Tensor) for e in column), f"Elements are not tensors: {column}"
-            fields.append(torch.cat(column, dim=0))
+            joined = _already_joined(column, shared_buffer)
+            fields.append(joined if joined is not None else torch.cat(column, dim=0))
         return tuple(fields)
     return first
 
@@ -224,7 +246,7 @@ class DynaFlowManager:
         # the caller's stream continues only after every nano-batch's last launch
         for event in events:
             event.wait()
-        return join_results(results, len(results))
+        return join_results(results, len(results), getattr(self.engine, "shared_output_buffer", None))
 
     # ------------------------------------------------- whole-schedule graphs
     def _wants_whole_graph(self, split: SplitConfig) -> bool:

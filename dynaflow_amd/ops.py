@@ -22,6 +22,7 @@ from __future__ import annotations
 
 import math
 import os
+import threading
 
 import torch
 
@@ -39,6 +40,8 @@ _lib.define("transpose_weight(Tensor w) -> Tensor")
 _lib.define("rope(Tensor t, Tensor cos, Tensor sin) -> Tensor")
 _lib.define("causal_attention(Tensor q, Tensor k, Tensor v) -> Tensor")
 _lib.define("linear_add(Tensor x, Tensor weight, Tensor residual) -> Tensor")
+_lib.define("linear_to_output(Tensor x, Tensor weight) -> Tensor")
+_lib.define("linear_add_to_output(Tensor x, Tensor weight, Tensor residual) -> Tensor")
 _lib.define(
     "decode_attention(Tensor qkv, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor slots, Tensor lengths, "
     "Tensor cos, Tensor sin, int q_heads, int kv_heads) -> Tensor"
@@ -119,7 +122,39 @@ def _plan_bf16(lib, M: int, N: int, K: int) -> tuple[int, int]:
     return variant.value, split_k.value
 
 
-def _linear_impl(x: torch.Tensor, weight: torch.Tensor, variant: int = -1, split_k_allowed: bool = True) -> torch.Tensor:
+# ------------------------------------------------------------ output rows
+# The engine may offer, for the sub-graph call that produces a nano-batch's share of the model output, the rows
+# of ONE buffer shared by all nano-batches; the ``*_to_output`` operators (what the lowering makes of the
+# projection whose result the sub-graph returns) write there, and the per-nano-batch results then need no
+# concatenation.  An offer holds for one operator call of the offering thread and is withdrawn by the engine
+# after the sub-graph call.
+_output_offer = threading.local()
+
+
+def offer_output_rows(provider) -> None:
+    """``provider(rows, cols, dtype, device) -> Tensor [rows, cols] | None`` for the next ``*_to_output`` call."""
+    _output_offer.provider = provider
+
+
+def withdraw_output_rows() -> None:
+    _output_offer.provider = None
+
+
+def _new_output(rows: int, cols: int, dtype: torch.dtype, device: torch.device, to_output: bool) -> torch.Tensor:
+    if to_output:
+        provider = getattr(_output_offer, "provider", None)
+        if provider is not None:
+            _output_offer.provider = None
+            given = provider(rows, cols, dtype, device)
+            if given is not None:
+                if tuple(given.shape) != (rows, cols) or given.dtype != dtype or not given.is_contiguous():
+                    raise RuntimeError("output rows offered to the operator do not fit its result")
+                return given
+    return torch.empty((rows, cols), dtype=dtype, device=device)
+
+
+def _linear_impl(x: torch.Tensor, weight: torch.Tensor, variant: int = -1, split_k_allowed: bool = True,
+                 to_output: bool = False) -> torch.Tensor:
     _require_device(x, weight)
     lib = _cabi.load()
     if weight.dim() != 2 or x.shape[-1] != weight.shape[1]:
@@ -128,7 +163,7 @@ def _linear_impl(x: torch.Tensor, weight: torch.Tensor, variant: int = -1, split
         raise RuntimeError(f"linear: dtype mismatch {x.dtype} vs {weight.dtype}")
     a, M, K, lda = _rows(x)
     w, N, _, ldw = _rows(weight)
-    out = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    out = _new_output(M, N, x.dtype, x.device, to_output)
     if M > 0:
         if x.dtype == torch.bfloat16:
             if variant == -2:
@@ -170,12 +205,15 @@ def _linear_fake(x, weight):
 
 _lib.impl("linear", lambda x, w: _linear_impl(x, w), "CUDA")
 _lib.impl("linear_variant", lambda x, w, v: _linear_impl(x, w, v), "CUDA")
+_lib.impl("linear_to_output", lambda x, w: _linear_impl(x, w, to_output=True), "CUDA")
 torch.library.register_fake("dynaflow_hip::linear", _linear_fake, lib=_lib)
+torch.library.register_fake("dynaflow_hip::linear_to_output", _linear_fake, lib=_lib)
 torch.library.register_fake("dynaflow_hip::linear_variant", lambda x, w, v: _linear_fake(x, w), lib=_lib)
 
 
 # ------------------------------------------------ projection + residual addition
-def _linear_add_impl(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+def _linear_add_impl(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor,
+                     to_output: bool = False) -> torch.Tensor:
     """``residual + x @ weight.T`` (bf16) in one launch, rounded like the separate linear and add kernels."""
     _require_device(x, weight, residual)
     lib = _cabi.load()
@@ -190,7 +228,7 @@ def _linear_add_impl(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tens
     r = residual.reshape(M, N)
     if r.stride(1) != 1 or r.stride(0) != N:
         r = r.contiguous()
-    out = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    out = _new_output(M, N, x.dtype, x.device, to_output)
     if M > 0:
         stream = _stream()
         _, split_k = _plan_bf16(lib, M, N, K)
@@ -210,7 +248,9 @@ def _linear_add_impl(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tens
 
 
 _lib.impl("linear_add", _linear_add_impl, "CUDA")
+_lib.impl("linear_add_to_output", lambda x, w, r: _linear_add_impl(x, w, r, to_output=True), "CUDA")
 torch.library.register_fake("dynaflow_hip::linear_add", lambda x, w, r: _linear_fake(x, w), lib=_lib)
+torch.library.register_fake("dynaflow_hip::linear_add_to_output", lambda x, w, r: _linear_fake(x, w), lib=_lib)
 
 
 # ------------------------------------------- gate/up projection + SiLU*mul epilogue
@@ -564,6 +604,8 @@ rope = torch.ops.dynaflow_hip.rope
 decode_attention = torch.ops.dynaflow_hip.decode_attention
 causal_attention = torch.ops.dynaflow_hip.causal_attention
 linear_add = torch.ops.dynaflow_hip.linear_add
+linear_to_output = torch.ops.dynaflow_hip.linear_to_output
+linear_add_to_output = torch.ops.dynaflow_hip.linear_add_to_output
 quant_fp8 = torch.ops.dynaflow_hip.quant_fp8
 silu_mul_quant_fp8 = torch.ops.dynaflow_hip.silu_mul_quant_fp8
 linear_fp8 = torch.ops.dynaflow_hip.linear_fp8

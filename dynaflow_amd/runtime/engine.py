@@ -45,12 +45,60 @@ def _is_symbolic(value: Any) -> bool:
     return isinstance(value, torch.SymInt)
 
 
+class _SharedOutput:
+    """Rows of one output buffer handed to the operator that ends each nano-batch (``ops.offer_output_rows``).
+
+    The buffer is allocated when the first operator asks, on the stream of the caller of the forward (whose
+    earlier work every nano-batch stream has waited for), with as many rows as the asking nano-batch's share
+    of the tokens implies; a nano-batch gets the rows at its token offset.
+    """
+
+    def __init__(self, module_name: str, split_config: SplitConfig, device: Any) -> None:
+        self.module_name = module_name
+        self.split = split_config
+        self.origin_stream = device.current_stream()
+        self.buffer: torch.Tensor | None = None
+
+    def offer(self, op: OperatorHandle) -> bool:
+        if op.module_name != self.module_name:
+            return False
+        from dynaflow_amd import ops
+
+        b = op.batch_idx
+        tokens, total = self.split.num_tokens[b], self.split.split_indices[-1]
+        first = self.split.split_indices[b]
+
+        def provider(rows: int, cols: int, dtype: torch.dtype, dev: torch.device) -> torch.Tensor | None:
+            if tokens <= 0 or rows % tokens:
+                return None
+            per_token = rows // tokens
+            if self.buffer is None:
+                with torch.cuda.stream(self.origin_stream):
+                    self.buffer = torch.empty((per_token * total, cols), dtype=dtype, device=dev)
+            buf = self.buffer
+            if buf.shape[1] != cols or buf.dtype != dtype or buf.shape[0] != per_token * total:
+                return None
+            buf.record_stream(torch.cuda.current_stream())
+            return buf[per_token * first: per_token * first + rows]
+
+        ops.offer_output_rows(provider)
+        return True
+
+    @staticmethod
+    def withdraw() -> None:
+        from dynaflow_amd import ops
+
+        ops.withdraw_output_rows()
+
+
 class DynaFlowEngine:
     """Runs a split ``GraphModule`` under a scheduler's control."""
 
     def __init__(self, graph_module: torch.fx.GraphModule, config: DynaFlowConfig) -> None:
         self.graph_module = graph_module
         self.config = config
+        #: the buffer that the last forward's nano-batches wrote their output rows into (or None)
+        self.shared_output_buffer: torch.Tensor | None = None
         self.max_tokens = int(config.knob("max_tokens", _DEFAULT_MAX_TOKENS))
         # static input buffers for graph replay: [nano-batch][placeholder index]
         self.input_buffers: list[dict[int, torch.Tensor]] = [
@@ -186,6 +234,37 @@ class DynaFlowEngine:
             _use_cudagraph=split_config.use_cudagraph,
         )
 
+    def _shared_output_for(self, split_config: SplitConfig, device: Any) -> "_SharedOutput | None":
+        """One buffer for the model output of all nano-batches, when the graph allows it: the graph returns the
+        result of its last sub-graph call as it is, that result is token-shaped, and no per-sub-graph graph or
+        capture-size padding stands between the operator and its output."""
+        if not device.is_gpu or split_config.is_dryrun or split_config.use_cudagraph:
+            return None
+        if not self.config.knob("shared_output", True):
+            return None
+        if list(split_config.num_tokens_padded) != list(split_config.num_tokens):
+            return None
+        output = self.nodes[-1]
+        if output.op != "output":
+            return None
+        producer = output.args[0]
+        if isinstance(producer, (tuple, list)) and len(producer) == 1:
+            producer = producer[0]                       # dynamo graphs return a one-element tuple
+        if not isinstance(producer, torch.fx.Node) or producer.op != "call_module" or len(producer.users) != 1:
+            return None
+        # what the sub-graph returns is recorded inside it (the call node itself carries no example value)
+        module = getattr(self.graph_module, producer.target)
+        inner = getattr(module, "gm", module)
+        if not isinstance(inner, torch.fx.GraphModule):
+            return None
+        returned = next(n for n in inner.graph.nodes if n.op == "output").args[0]
+        if not isinstance(returned, torch.fx.Node):
+            return None
+        example = returned.meta.get("example_value", None)
+        if not isinstance(example, torch.Tensor) or example.dim() < 1 or not _is_symbolic(example.shape[0]):
+            return None
+        return _SharedOutput(producer.target, split_config, device)
+
     # ------------------------------------------------------------------ dry-run
     def dryrun(
         self, args: tuple, kwargs: dict, split_config: SplitConfig
@@ -316,6 +395,8 @@ class DynaFlowEngine:
                 self._execute_non_module(node, b, args, env, split_config)
                 queue.popleft()
 
+        shared_output = self._shared_output_for(split_config, device)
+
         # Inputs of every nano-batch are bound up front, on the caller's stream.
         for b in range(lanes):
             queue = todo[b]
@@ -379,7 +460,12 @@ class DynaFlowEngine:
                 for i, op in enumerate(operators):
                     with device.range(f"op_{op.module_name}_{op.batch_idx}"), set_op_handle(op):
                         module = getattr(self.graph_module, op.module_name)
-                        outputs.append(module(*call_pos[i], **call_kw[i]))
+                        offered = shared_output.offer(op) if shared_output is not None else False
+                        try:
+                            outputs.append(module(*call_pos[i], **call_kw[i]))
+                        finally:
+                            if offered:
+                                shared_output.withdraw()
 
             for op, value in zip(operators, outputs):
                 b = op.batch_idx
@@ -397,4 +483,5 @@ class DynaFlowEngine:
                     await run_inline_until_op(b)
             finished.set()
 
+        self.shared_output_buffer = shared_output.buffer if shared_output is not None else None
         return results, tail_events

@@ -214,3 +214,26 @@ def test_scheduler_that_returns_early_leaves_engine_waiting(host_device):
 
     with pytest.raises(asyncio.TimeoutError):
         asyncio.run(bounded())
+
+
+def test_join_results_skips_the_copy_for_consecutive_rows_of_one_buffer():
+    from dynaflow_amd.manager import join_results
+
+    buf = torch.arange(24.0).reshape(6, 4).clone()
+    parts = {0: buf[0:2], 1: buf[2:5], 2: buf[5:6]}
+    joined = join_results(parts, 3, buf)
+    assert joined.data_ptr() == buf.data_ptr() and torch.equal(joined, buf)
+    # views with more dimensions (sequences x positions x hidden) of the same rows
+    joined3 = join_results({0: buf[0:4].view(2, 2, 4), 1: buf[4:6].view(1, 2, 4)}, 2, buf)
+    assert joined3.data_ptr() == buf.data_ptr() and joined3.shape == (3, 2, 4)
+    # a one-element tuple per nano-batch (what a dynamo graph returns)
+    (field,) = join_results({0: (buf[0:3],), 1: (buf[3:6],)}, 2, buf)
+    assert field.data_ptr() == buf.data_ptr()
+    # rows of a buffer that is not the engine's own (say, views of an input) are copied like torch.cat does
+    assert join_results({0: buf[0:3], 1: buf[3:6]}, 2).data_ptr() != buf.data_ptr()
+    # anything else is concatenated: a gap, a wrong order, separate tensors, part of a larger buffer
+    for parts in ({0: buf[0:2], 1: buf[3:6]}, {0: buf[3:6], 1: buf[0:3]}, {0: buf[0:3].clone(), 1: buf[3:6].clone()},
+                  {0: buf[0:2], 1: buf[2:4]}):
+        joined = join_results(parts, 2, buf)
+        assert joined.data_ptr() != buf.data_ptr()
+        assert torch.equal(joined, torch.cat([parts[0], parts[1]], dim=0))

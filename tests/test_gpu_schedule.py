@@ -57,7 +57,7 @@ def test_subgraphs_run_on_hip_operators():
     for name in ("submod_0", "submod_1"):
         backend = manager.graph_module.__dict__[name]
         targets = [n.target for n in backend.callable_dynamic.graph.nodes if n.op == "call_function"]
-        assert all(t in (ops.linear, ops.silu_mul) for t in targets), targets
+        assert all(t in (ops.linear, ops.linear_to_output, ops.silu_mul) for t in targets), targets
 
 
 def test_config1_fp32_matches_cpu_reference_path():
@@ -102,6 +102,31 @@ def test_config2_full_size_properties():
     # a second overlapped run is bit-identical (no race between the streams)
     y2, _ = run(manager, compiled, xg, 4096)
     assert torch.equal(y, y2)
+
+
+def test_nano_batch_outputs_land_in_one_buffer(monkeypatch):
+    """The down projection of every nano-batch writes its rows of one output buffer: the forward ends without a
+    concatenation, and the result has the bits of the schedule that allocates per nano-batch and concatenates."""
+    manager, compiled, xg, _ = build(512, 512, 1408, torch.bfloat16, splits=2)
+    plain_manager, plain, xp, _ = build(512, 512, 1408, torch.bfloat16, splits=2, shared_output=False)
+    want, _ = run(plain_manager, plain, xp, 512)
+    real_cat = torch.cat
+
+    def no_cat(*args, **kwargs):
+        raise AssertionError("the forward concatenated its nano-batch outputs")
+
+    monkeypatch.setattr(torch, "cat", no_cat)
+    got, split = run(manager, compiled, xg, 512)
+    monkeypatch.setattr(torch, "cat", real_cat)
+    assert split.num_nano_batches == 2
+    assert got.shape == want.shape and torch.equal(got, want)
+    # ragged split (3 nano-batches of 171, 171, 170 tokens)
+    manager3, compiled3, x3, (x, wg, wu, wd) = build(512, 512, 1408, torch.bfloat16, splits=3)
+    monkeypatch.setattr(torch, "cat", no_cat)
+    got3, split3 = run(manager3, compiled3, x3, 512)
+    monkeypatch.setattr(torch, "cat", real_cat)
+    assert split3.num_nano_batches == 3
+    assert rel_err(got3.float(), mlp.mlp_schedule(x, wg, wu, wd, split3.split_indices).float()) < TOL["bf16"]
 
 
 def test_serialized_schedule_is_bit_identical_to_overlapped():
@@ -316,7 +341,7 @@ def test_fused_silu_epilogue_schedule():
     head = manager.graph_module.__dict__["submod_0"].callable_dynamic
     tail = manager.graph_module.__dict__["submod_1"].callable_dynamic
     assert [n.target for n in head.graph.nodes if n.op == "call_function"] == [ops.gate_up_silu]
-    assert [n.target for n in tail.graph.nodes if n.op == "call_function"] == [ops.linear]
+    assert [n.target for n in tail.graph.nodes if n.op == "call_function"] == [ops.linear_to_output]
     y, split = run(manager, compiled, xg, 1024)
     assert manager.engine.issue_trace == [("submod_0", 0), ("submod_1", 0), ("submod_0", 1), ("submod_1", 1)]
     want = mlp.mlp_fp32_from(x, wg, wu, wd)
@@ -366,10 +391,13 @@ def test_decoder_layer_attention_beside_mlp_small():
     mlp_graph = manager.graph_module.__dict__[names[1]].callable_dynamic
     targets = [n.target for n in mlp_graph.graph.nodes if n.op == "call_function"]
     assert ops.rms_norm in targets and ops.silu_mul in targets
-    assert targets.count(ops.linear) == 2 and targets.count(ops.linear_add) == 1   # down projection + residual
+    # down projection + residual in one launch; as the value the sub-graph returns it may write into offered rows
+    assert targets.count(ops.linear) == 2
+    assert targets.count(ops.linear_add) + targets.count(ops.linear_add_to_output) == 1
     attn_targets = [n.target for n in manager.graph_module.__dict__[names[0]].callable_dynamic.graph.nodes
                     if n.op == "call_function"]
-    assert attn_targets.count(ops.linear) == 3 and attn_targets.count(ops.linear_add) == 1
+    assert attn_targets.count(ops.linear) == 3
+    assert attn_targets.count(ops.linear_add) + attn_targets.count(ops.linear_add_to_output) == 1
     assert ops.rms_norm in attn_targets
     assert attn_targets.count(ops.rope) == 2
     with torch.no_grad():
