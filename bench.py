@@ -114,6 +114,27 @@ def time_steps(torch, manager, compiled, x, steps, warmup, use_graph):
     return (t1 - t0) * 1e3 / steps, y
 
 
+def gpu_time_of_steps(torch, manager, compiled, x, steps):
+    """GPU-side duration of one eagerly issued step (median over ``steps``, ms): the GPU is kept busy with a
+    spin kernel while the host issues the whole step behind it, so the interval between the two events holds the
+    step's kernels back to back and none of the host's issue time."""
+    spin_cycles = 8_000_000   # about 4 ms: longer than the host needs to issue a step
+    times = []
+    with torch.no_grad():
+        for _ in range(steps):
+            manager.prepare(TOKENS, [TOKENS], use_cudagraph=False)
+            start = torch.cuda.Event(enable_timing=True)
+            stop = torch.cuda.Event(enable_timing=True)
+            torch.cuda._sleep(spin_cycles)
+            start.record()
+            compiled(x)
+            stop.record()
+            stop.synchronize()
+            times.append(start.elapsed_time(stop))
+    times.sort()
+    return times[len(times) // 2]
+
+
 def time_kernel(torch, fn, iters, warmup=20):
     """Average duration of one launch, from HIP events on the stream it is launched on."""
     for _ in range(warmup):
@@ -479,6 +500,7 @@ def main() -> int:
     m_ser, c_ser = build_path(torch, x, weights, serialize=True)
     ms_serial, y_serial = time_steps(torch, m_ser, c_ser, x, args.steps, args.warmup, use_graph=False)
     y_serial = y_serial.clone()
+    ms_serial_gpu = gpu_time_of_steps(torch, m_ser, c_ser, x, min(args.steps, 20))
     m_ovl, c_ovl = build_path(torch, x, weights, whole_graph=True)
     ms_eager, y_eager = time_steps(torch, m_ovl, c_ovl, x, args.steps, args.warmup, use_graph=False)
     y_eager = y_eager.clone()
@@ -490,6 +512,7 @@ def main() -> int:
     m_fs, c_fs = build_path(torch, x, weights, serialize=True, fuse_silu_epilogue=True)
     ms_fused_serial, yf_serial = time_steps(torch, m_fs, c_fs, x, args.steps, args.warmup, use_graph=False)
     yf_serial = yf_serial.clone()
+    ms_fused_serial_gpu = gpu_time_of_steps(torch, m_fs, c_fs, x, min(args.steps, 20))
     m_fo, c_fo = build_path(torch, x, weights, whole_graph=True, fuse_silu_epilogue=True)
     ms_fused_graph, yf_graph = time_steps(torch, m_fo, c_fo, x, args.steps, args.warmup, use_graph=True)
     fused_identical = bool(torch.equal(yf_serial, yf_graph))
@@ -534,16 +557,20 @@ def main() -> int:
         },
         "overlap": {
             "serialized_ms": ms_serial,
+            "serialized_gpu_side_ms": ms_serial_gpu,
             "overlapped_eager_ms": ms_eager,
             "overlapped_graph_ms": ms_graph,
             "speedup_eager_vs_serialized": ms_serial / ms_eager,
             "speedup_graph_vs_serialized": ms_serial / ms_graph,
+            "speedup_graph_vs_serialized_gpu_side": ms_serial_gpu / ms_graph,
             "outputs_bit_identical": identical,
         },
         "silu_mul_as_gemm_epilogue": {
             "serialized_ms": ms_fused_serial,
+            "serialized_gpu_side_ms": ms_fused_serial_gpu,
             "overlapped_graph_ms": ms_fused_graph,
             "speedup_graph_vs_serialized": ms_fused_serial / ms_fused_graph,
+            "speedup_graph_vs_serialized_gpu_side": ms_fused_serial_gpu / ms_fused_graph,
             "outputs_bit_identical": fused_identical,
             "rel_err_vs_fp32_oracle_sampled_rows": rel_err_fused,
         },
