@@ -282,7 +282,9 @@ def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False) -> tuple[
     output = next(n for n in graph.nodes if n.op == "output")
     returned = output.args[0]
     if isinstance(returned, fx.Node) and returned.op == "call_function" and len(returned.users) == 1:
-        into = {ops.linear: ops.linear_to_output, ops.linear_add: ops.linear_add_to_output}.get(returned.target)
+        packet = getattr(returned.target, "overloadpacket", returned.target)   # traced calls carry the overload
+        into = {ops.linear: ops.linear_to_output, ops.linear_add: ops.linear_add_to_output,
+                ops.linear_fp8: ops.linear_fp8_to_output}.get(packet)
         if into is not None and not returned.kwargs:
             returned.target = into
             stats["to_output"] = 1

@@ -50,6 +50,7 @@ _lib.define("quant_fp8(Tensor x) -> (Tensor, Tensor)")
 _lib.define("silu_mul_quant_fp8(Tensor gate, Tensor up) -> (Tensor, Tensor)")
 _lib.define("linear_fp8(Tensor x_q, Tensor w_q, Tensor x_scale, Tensor w_scale) -> Tensor")
 _lib.define("linear_fp8_variant(Tensor x_q, Tensor w_q, Tensor x_scale, Tensor w_scale, int variant) -> Tensor")
+_lib.define("linear_fp8_to_output(Tensor x_q, Tensor w_q, Tensor x_scale, Tensor w_scale) -> Tensor")
 
 FP8_DTYPE = torch.float8_e4m3fn
 FP8_MAX = 448.0
@@ -547,7 +548,7 @@ def _silu_mul_quant_fp8_impl(gate: torch.Tensor, up: torch.Tensor):
     return q.view(gate.shape), scale
 
 
-def _linear_fp8_impl(x_q, w_q, x_scale, w_scale, variant: int = -1):
+def _linear_fp8_impl(x_q, w_q, x_scale, w_scale, variant: int = -1, to_output: bool = False):
     _require_device(x_q, w_q, x_scale, w_scale)
     lib = _cabi.load()
     if x_q.dtype != FP8_DTYPE or w_q.dtype != FP8_DTYPE:
@@ -558,7 +559,7 @@ def _linear_fp8_impl(x_q, w_q, x_scale, w_scale, variant: int = -1):
     w, N, Kw, ldw = _rows(w_q)
     if K != Kw or w_scale.numel() != N or x_scale.numel() != 1:
         raise RuntimeError("linear_fp8: shape mismatch")
-    out = torch.empty((M, N), dtype=torch.bfloat16, device=x_q.device)
+    out = _new_output(M, N, torch.bfloat16, x_q.device, to_output)
     if M > 0:
         rc = lib.dfhip_gemm_fp8_nt_variant(
             a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), N,
@@ -571,7 +572,8 @@ def _linear_fp8_impl(x_q, w_q, x_scale, w_scale, variant: int = -1):
 _lib.impl("quant_fp8", _quant_fp8_impl, "CUDA")
 _lib.impl("silu_mul_quant_fp8", _silu_mul_quant_fp8_impl, "CUDA")
 _lib.impl("linear_fp8", lambda x_q, w_q, xs, ws: _linear_fp8_impl(x_q, w_q, xs, ws), "CUDA")
-_lib.impl("linear_fp8_variant", _linear_fp8_impl, "CUDA")
+_lib.impl("linear_fp8_variant", lambda x_q, w_q, xs, ws, v: _linear_fp8_impl(x_q, w_q, xs, ws, v), "CUDA")
+_lib.impl("linear_fp8_to_output", lambda x_q, w_q, xs, ws: _linear_fp8_impl(x_q, w_q, xs, ws, to_output=True), "CUDA")
 torch.library.register_fake(
     "dynaflow_hip::quant_fp8",
     lambda x: (x.new_empty(x.shape, dtype=FP8_DTYPE), x.new_empty((1,), dtype=torch.float32)),
@@ -584,6 +586,11 @@ torch.library.register_fake(
 )
 torch.library.register_fake(
     "dynaflow_hip::linear_fp8",
+    lambda x_q, w_q, xs, ws: x_q.new_empty((*x_q.shape[:-1], w_q.shape[0]), dtype=torch.bfloat16),
+    lib=_lib,
+)
+torch.library.register_fake(
+    "dynaflow_hip::linear_fp8_to_output",
     lambda x_q, w_q, xs, ws: x_q.new_empty((*x_q.shape[:-1], w_q.shape[0]), dtype=torch.bfloat16),
     lib=_lib,
 )
@@ -610,3 +617,4 @@ quant_fp8 = torch.ops.dynaflow_hip.quant_fp8
 silu_mul_quant_fp8 = torch.ops.dynaflow_hip.silu_mul_quant_fp8
 linear_fp8 = torch.ops.dynaflow_hip.linear_fp8
 linear_fp8_variant = torch.ops.dynaflow_hip.linear_fp8_variant
+linear_fp8_to_output = torch.ops.dynaflow_hip.linear_fp8_to_output
