@@ -237,3 +237,78 @@ def test_join_results_skips_the_copy_for_consecutive_rows_of_one_buffer():
         joined = join_results(parts, 2, buf)
         assert joined.data_ptr() != buf.data_ptr()
         assert torch.equal(joined, torch.cat([parts[0], parts[1]], dim=0))
+
+
+_REFERENCE_STYLE_POLICY = '''
+"""A policy file written against the reference package's import names (not this build's)."""
+from typing_extensions import override
+
+from dynaflow.config import DynaFlowConfig
+from dynaflow.interface import ExecutionContext, InputInfo, OpSchedulerBase, SplitConfig
+from dynaflow.matching import MatchingRule, Op
+from dynaflow.utils import pack_tokens
+
+
+class TwoWay(OpSchedulerBase):
+    def __init__(self, config: DynaFlowConfig) -> None:
+        super().__init__(policy_name="two_way")
+        self.capture_sizes = config.cudagraph_config.capture_sizes
+
+    @override
+    def get_split_rules(self) -> list[MatchingRule]:
+        return [MatchingRule(condition=(Op("silu"), Op("mul"), Op("linear")))]
+
+    @override
+    def get_tag_rules(self) -> dict[MatchingRule, set[str]]:
+        return {MatchingRule(condition=Op("mul")): {"tail"}}
+
+    @override
+    def get_split_config(self, input_info: InputInfo, use_cudagraph: bool = False) -> SplitConfig:
+        total = sum(input_info.num_tokens)
+        left = total // 2
+        padded, fits = pack_tokens(left, self.capture_sizes)
+        assert fits and padded >= left
+        return SplitConfig(num_nano_batches=2, batch_sizes=[1, 1], batch_indices=[0, 1, 2],
+                           num_tokens=[left, total - left], num_tokens_padded=[left, total - left],
+                           split_indices=[0, left, total], is_dryrun=False, use_cudagraph=False)
+
+    @override
+    async def schedule(self, context: ExecutionContext) -> None:
+        live = [0, 1]
+        while live:
+            for b in list(live):
+                op = await context.pop(b)
+                if op is None:
+                    live.remove(b)
+                    continue
+                await context.execute((op,))
+'''
+
+
+def test_policy_file_written_against_the_reference_package_names_runs_unmodified(host_device, tmp_path):
+    import sys
+
+    import dynaflow_amd
+
+    path = tmp_path / "two_way_policy.py"
+    path.write_text(_REFERENCE_STYLE_POLICY)
+    dynaflow_amd.install_as_dynaflow()
+    try:
+        import dynaflow.executor.cudagraph as graphs  # the reference's module name for the graph wrapper
+
+        assert hasattr(graphs, "CUDAGraphWrapper")
+        cfg = DynaFlowConfig(f"{path}:TwoWay", 2, InductorConfig(enabled=False),
+                             CUDAGraphConfig(enabled=False, capture_sizes=[64, 128]),
+                             {"min_nano_split_tokens": 8, "dump_graph": False})
+        model, manager, compiled, x = compile_mlp(cfg, tokens=96)
+        assert type(manager.scheduler).__name__ == "TwoWay" and manager.scheduler.policy_name == "two_way"
+        split = manager.prepare(96, [96])
+        assert split.split_indices == [0, 48, 96]
+        with torch.no_grad():
+            got = compiled(x)
+            want = model(x)
+        assert torch.allclose(got, want, atol=1e-6)
+        assert manager.engine.issue_trace == [("submod_0", 0), ("submod_0", 1), ("submod_1", 0), ("submod_1", 1)]
+    finally:
+        for name in [n for n in sys.modules if n == "dynaflow" or n.startswith("dynaflow.")]:
+            del sys.modules[name]
