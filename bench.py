@@ -368,7 +368,8 @@ def decode_config(torch, steps, warmup, layers=32):
     half = seqs // 2
     results = {}
     for name, knobs, graphs in (("serialized_eager", {"serialize": True}, False), ("overlapped_eager", {}, False),
-                                ("overlapped_sub_graph_replay", {}, True)):
+                                ("overlapped_sub_graph_replay", {}, True),
+                                ("stream_per_nano_batch_sub_graph_replay", {"streams": "by_nano_batch"}, True)):
         extra = {"min_nano_split_tokens": 1, "dump_graph": False, "max_tokens": seqs, "fuse_silu_epilogue": True}
         extra.update(knobs)
         cfg = DynaFlowConfig("dynaflow_amd.schedulers:DecoderOverlapScheduler", 2, InductorConfig(enabled=True),
@@ -408,7 +409,8 @@ def decode_config(torch, steps, warmup, layers=32):
         "config": {"workload": f"decode step over {layers} Llama-3-8B-shaped layers, {seqs} single-token queries, "
                                f"{capacity} cached positions per sequence, 2 nano-batches of {half}; whole-schedule "
                                "graph capture is switched off for this model, the best of the eager two-stream "
-                               "schedule and per-sub-graph graph replay is reported"},
+                               "schedule and per-sub-graph graph replay (streams by sub-graph kind or one per "
+                               "nano-batch) is reported"},
         "timings": results,
         "roofline": {"bound": "hbm", "achieved": (weight_bytes + kv_bytes) / (best * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -36,9 +36,12 @@ decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
                         const uint16_t* __restrict__ vc, const int32_t* __restrict__ slots,
                         const int32_t* __restrict__ lengths, uint16_t* __restrict__ out, int64_t ld_out,
                         int kv_heads, int group, int num_slots, int capacity, float scale_log2) {
-  __shared__ float o_lds[4][MAX_GROUP][HD];
-  __shared__ float m_lds[4][MAX_GROUP];
-  __shared__ float l_lds[4][MAX_GROUP];
+  // partial results of the four waves, sized by the launch for the real group (a workgroup that asks for
+  // little LDS leaves room for a GEMM workgroup of the other nano-batch on the same CU)
+  extern __shared__ __attribute__((aligned(16))) float combine_lds[];
+  float* const o_lds = combine_lds;                       // [4][group][HD]
+  float* const m_lds = combine_lds + 4 * group * HD;      // [4][group]
+  float* const l_lds = m_lds + 4 * group;                 // [4][group]
   const int t = blockIdx.x / kv_heads, kvh = blockIdx.x - t * kv_heads;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hq = lane & 15, g = lane >> 4;
@@ -148,25 +151,25 @@ decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
     const int h = 4 * g + r;
     if (h < group) {
 #pragma unroll
-      for (int nb = 0; nb < 8; ++nb) o_lds[wave][h][nb * 16 + hq] = o[nb][r];
+      for (int nb = 0; nb < 8; ++nb) o_lds[(wave * group + h) * HD + nb * 16 + hq] = o[nb][r];
     }
   }
-  if (g == 0) {
-    m_lds[wave][hq] = m;
-    l_lds[wave][hq] = l;
+  if (g == 0 && hq < group) {
+    m_lds[wave * group + hq] = m;
+    l_lds[wave * group + hq] = l;
   }
   __syncthreads();
   for (int idx = tid; idx < group * HD; idx += DEC_THREADS) {
     const int h = idx >> 7, dim = idx & (HD - 1);
-    float mm = m_lds[0][h];
+    float mm = m_lds[h];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) mm = fmaxf(mm, m_lds[w][h]);
+    for (int w = 1; w < 4; ++w) mm = fmaxf(mm, m_lds[w * group + h]);
     float num = 0.0f, den = 0.0f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      const float f = exp2f(m_lds[w][h] - mm);   // 0 for a wave that had no chunk (m = -inf)
-      num += o_lds[w][h][dim] * f;
-      den += l_lds[w][h] * f;
+      const float f = exp2f(m_lds[w * group + h] - mm);   // 0 for a wave that had no chunk (m = -inf)
+      num += o_lds[(w * group + h) * HD + dim] * f;
+      den += l_lds[w * group + h] * f;
     }
     out_row[idx] = static_cast<uint16_t>(f32_to_bf16_bits(num / den));
   }
@@ -243,10 +246,12 @@ extern "C" int dfhip_decode_attention_bf16(const void* q, int64_t ld_q, const vo
   if (ld_q % 8 || !dfhip_aligned16(q) || !dfhip_aligned16(k_cache) || !dfhip_aligned16(v_cache))
     return DFHIP_ERR_BAD_ALIGNMENT;
   const float scale_log2 = scale * 1.4426950408889634f;
-  hipLaunchKernelGGL(decode_attention_kernel, dim3(T * kv_heads), dim3(DEC_THREADS), 0,
+  const int group = q_heads / kv_heads;
+  const size_t combine_bytes = (size_t)4 * group * (HD + 2) * sizeof(float);
+  hipLaunchKernelGGL(decode_attention_kernel, dim3(T * kv_heads), dim3(DEC_THREADS), combine_bytes,
                      static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(q), ld_q,
                      static_cast<const uint16_t*>(k_cache), static_cast<const uint16_t*>(v_cache), slots, lengths,
-                     static_cast<uint16_t*>(out), ld_out, kv_heads, q_heads / kv_heads, num_slots, capacity,
+                     static_cast<uint16_t*>(out), ld_out, kv_heads, group, num_slots, capacity,
                      scale_log2);
   return dfhip_check_launch();
 }

@@ -34,6 +34,13 @@ class StaggeredScheduler(OpSchedulerBase):
         device = get_device()
         self.comm_stream = device.new_stream("side")
         self.comp_stream = device.new_stream("main")
+        # "by_kind": tagged sub-graphs on the side stream, the others on the main one (the reference's policies);
+        # "by_nano_batch": every nano-batch keeps one stream for its whole chain, so that sub-graphs of the same
+        # kind of different nano-batches can run side by side as well (with the staggered order they are one
+        # sub-graph apart)
+        self.stream_policy: str = config.knob("streams", "by_kind")
+        if self.stream_policy not in ("by_kind", "by_nano_batch"):
+            raise ValueError(f"unknown stream policy {self.stream_policy!r}")
 
     def get_split_rules(self) -> list[MatchingRule]:
         return self._split_rules
@@ -45,6 +52,8 @@ class StaggeredScheduler(OpSchedulerBase):
         return equal_n_way(input_info, use_cudagraph, self.num_nano_batches, self.min_nano_split_tokens)
 
     def _stream_for(self, op):
+        if self.stream_policy == "by_nano_batch" and self.comm_stream is not self.comp_stream:
+            return self.comm_stream if op.batch_idx % 2 else self.comp_stream
         return self.comm_stream if self.side_tag in op.tag else self.comp_stream
 
     async def _issue(self, context: ExecutionContext, op) -> None:

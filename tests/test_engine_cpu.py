@@ -312,3 +312,21 @@ def test_policy_file_written_against_the_reference_package_names_runs_unmodified
     finally:
         for name in [n for n in sys.modules if n == "dynaflow" or n.startswith("dynaflow.")]:
             del sys.modules[name]
+
+
+def test_one_stream_per_nano_batch_policy(host_device):
+    """``streams="by_nano_batch"``: every launch of nano-batch 0 on the main stream, of nano-batch 1 on the side
+    stream, whatever the sub-graph's tag; the issue order stays the staggered one and the result the same."""
+    cfg = make_config(2, streams="by_nano_batch")
+    model, manager, compiled, x = compile_mlp(cfg, tokens=96)
+    manager.prepare(96, [96])
+    host_device.log.clear()
+    with torch.no_grad():
+        y = compiled(x)
+    torch.testing.assert_close(y, model(x), rtol=0, atol=0)
+    ranges = [(e[1], e[2]) for e in host_device.log if e[0] == "range"]
+    launches = [(name.rsplit("_", 1)[0][3:], int(name.rsplit("_", 1)[1]), stream) for name, stream in ranges]
+    assert launches == [("submod_0", 0, "main"), ("submod_1", 0, "main"), ("submod_0", 1, "side"),
+                        ("submod_1", 1, "side")]
+    with pytest.raises(ValueError):
+        MLPOverlapScheduler(make_config(2, streams="per_kernel"))

@@ -120,7 +120,7 @@ def test_decode_attention_full_size_properties(ops):
     assert torch.equal(const, torch.full_like(const, 0.375))
 
 
-def build_decode(T, whole_graph, sub_graphs=False, **over):
+def build_decode(T, whole_graph, sub_graphs=False, knobs=None, **over):
     from dynaflow_amd.backend import make_backend
     from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
     from dynaflow_amd.decode import DecodeModel
@@ -142,7 +142,7 @@ def build_decode(T, whole_graph, sub_graphs=False, **over):
     cfg = DynaFlowConfig("dynaflow_amd.schedulers:DecoderOverlapScheduler", 2, InductorConfig(enabled=True),
                          CUDAGraphConfig(enabled=sub_graphs, capture_sizes=[T // 2, T]),
                          {"min_nano_split_tokens": 1, "dump_graph": False, "whole_graph": whole_graph,
-                          "max_tokens": T})
+                          "max_tokens": T, **(knobs or {})})
     manager = DynaFlowManager()
     torch._dynamo.reset()
     dev = [t.cuda() for t in (ids, slots, lengths)]
@@ -244,10 +244,12 @@ def test_decode_attention_under_graph_capture(ops):
     assert torch.equal(out, want) and not torch.equal(out, eager)
 
 
-def test_decode_schedule_with_sub_graph_replay():
+@pytest.mark.parametrize("streams", ["by_kind", "by_nano_batch"])
+def test_decode_schedule_with_sub_graph_replay(streams):
     """Per-sub-graph graphs (the reference's mechanism) on the decode model at shapes where the projections
     run on the weight-streaming kernel with K split: capture in a dry-run at the nano-batch size, then the
-    scheduled forward replays the graphs; every replay equals the eager two-stream result."""
+    scheduled forward replays the graphs; every replay equals the eager two-stream result - with the streams
+    chosen by sub-graph kind (attention / MLP) and with one stream per nano-batch."""
     T = 32
     over = dict(layers=2, hidden=1024, heads=8, kv_heads=2, inter=2048)
     print("decode sub-graph replay: eager model", flush=True)
@@ -257,7 +259,8 @@ def test_decode_schedule_with_sub_graph_replay():
         eager = compiled(*dev).clone()
         torch.cuda.synchronize()
     print("decode sub-graph replay: graph model", flush=True)
-    manager, compiled, dev, host2, model2, _, _ = build_decode(T, whole_graph=False, sub_graphs=True, **over)
+    manager, compiled, dev, host2, model2, _, _ = build_decode(T, whole_graph=False, sub_graphs=True,
+                                                               knobs={"streams": streams}, **over)
     half = T // 2
     with torch.no_grad():
         print("decode sub-graph replay: dry-run capture", flush=True)
