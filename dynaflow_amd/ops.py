@@ -83,31 +83,45 @@ def _require_device(*tensors: torch.Tensor) -> None:
 
 
 # ---------------------------------------------------------------- linear
-#: split-K workspaces, one per (device, stream): launches on one stream run one after the
-#: other, launches on different streams may overlap and must not share arrival counters
-_splitk_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+#: split-K workspaces.  Inside a DynaFlow launch: one per (device, nano-batch) - the launches of one nano-batch
+#: are chained one after the other whatever streams they run on, different nano-batches may overlap and must
+#: not share arrival counters.  Outside: one per (device, stream).
+_splitk_workspaces: dict[tuple, torch.Tensor] = {}
+#: workspaces that were replaced by larger ones: captured graphs may still point at them
+_retired_workspaces: list[torch.Tensor] = []
 #: split K for shapes with too few tiles (DYNAFLOW_SPLIT_K=0 switches it off)
 SPLIT_K_ENABLED = os.environ.get("DYNAFLOW_SPLIT_K", "1") != "0"
 
 
 def _zeroed_workspace(cache: dict, device: torch.device, stream: int, nbytes: int, clear: int = 65536) -> torch.Tensor:
-    """A per-(device, stream) scratch buffer whose first ``clear`` bytes are zero at first use.
+    """A scratch buffer whose first ``clear`` bytes are zero at first use, kept for the life of the process.
 
-    The kernels that use these buffers (split-K arrival counters) leave them zero.
+    The kernels that use these buffers (split-K arrival counters) leave them zero, so a buffer made by an
+    eager launch (the warm-up that precedes every capture) serves the captured launches of the same
+    nano-batch as it is: no allocation and no clearing inside the graph.
     """
-    key = (device.index or 0, stream)
+    from dynaflow_amd.interface import OperatorHandle
+    from dynaflow_amd.runtime.env import peek_op_handle
+
+    handle = peek_op_handle()
+    if isinstance(handle, OperatorHandle):
+        key = (device.index or 0, "nano-batch", handle.batch_idx)
+    else:
+        key = (device.index or 0, "stream", stream)
     ws = cache.get(key)
-    if torch.cuda.is_current_stream_capturing() and (ws is None or ws.numel() < nbytes):
-        # A capture on a stream of its own (per-sub-graph graphs): the buffer comes from the graph's
-        # memory pool and its start is zeroed by a fill kernel that is part of the graph - no memset
-        # node.  Graphs of one pool replay one after the other, so they may share.
+    if ws is not None and ws.numel() >= nbytes:
+        return ws
+    if torch.cuda.is_current_stream_capturing():
+        # No buffer from an eager launch to fall back on: this one comes from the graph's memory pool and its
+        # start is zeroed by a fill kernel that is part of the graph (a kernel, not a memset node).
         ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
         rc = _cabi.load().dfhip_fill_u32(ws.data_ptr(), 0, min(nbytes, clear) // 4, stream)
         _cabi.check("dfhip_fill_u32", rc)
         return ws
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
-        cache[key] = ws
+    if ws is not None:
+        _retired_workspaces.append(ws)
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+    cache[key] = ws
     return ws
 
 
