@@ -68,7 +68,22 @@ def parse_args():
     p.add_argument("--decoder", action="store_true",
                    help="measure the full Llama-3-8B-shaped decoder layer (prefill 8 x 2048, attention of one "
                         "nano-batch beside the MLP of the other) instead of the headline configuration")
+    p.add_argument("--knob", action="append", default=[], metavar="NAME=VALUE",
+                   help="extra entry of DynaFlowConfig.additional_config for every mode of the run (value read as "
+                        "JSON when it parses, else as a string), e.g. --knob streams=by_nano_batch")
     return p.parse_args()
+
+
+EXTRA_KNOBS: dict = {}
+
+
+def read_knobs(pairs):
+    for pair in pairs:
+        name, _, value = pair.partition("=")
+        try:
+            EXTRA_KNOBS[name] = json.loads(value)
+        except ValueError:
+            EXTRA_KNOBS[name] = value
 
 
 def build_path(torch, x, weights, **knobs):
@@ -83,7 +98,7 @@ def build_path(torch, x, weights, **knobs):
         model.gate_proj.weight.copy_(wg)
         model.up_proj.weight.copy_(wu)
         model.down_proj.weight.copy_(wd)
-    extra = {"min_nano_split_tokens": 64, "num_nano_batches": SPLITS, "dump_graph": False}
+    extra = {"min_nano_split_tokens": 64, "num_nano_batches": SPLITS, "dump_graph": False, **EXTRA_KNOBS}
     extra.update(knobs)
     cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", SPLITS, InductorConfig(enabled=True),
                          CUDAGraphConfig(enabled=False, capture_sizes=[TOKENS]), extra)
@@ -241,7 +256,7 @@ def fp8_config(torch, steps, warmup):
     del parts
     results = {}
     for name, knobs in (("serialized", {"serialize": True}), ("overlapped", {"whole_graph": True})):
-        extra = {"min_nano_split_tokens": 64, "num_nano_batches": splits, "dump_graph": False}
+        extra = {"min_nano_split_tokens": 64, "num_nano_batches": splits, "dump_graph": False, **EXTRA_KNOBS}
         extra.update(knobs)
         cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", splits, InductorConfig(enabled=True),
                              CUDAGraphConfig(enabled=False, capture_sizes=[tokens]), extra)
@@ -305,7 +320,7 @@ def decoder_config(torch, steps, warmup):
     results = {}
     for name, knobs in (("serialized", {"serialize": True}), ("overlapped", {"whole_graph": True}),
                         ("overlapped_fused_silu", {"whole_graph": True, "fuse_silu_epilogue": True})):
-        extra = {"min_nano_split_tokens": 64, "dump_graph": False}
+        extra = {"min_nano_split_tokens": 64, "dump_graph": False, **EXTRA_KNOBS}
         extra.update(knobs)
         cfg = DynaFlowConfig("dynaflow_amd.schedulers:DecoderOverlapScheduler", 2, InductorConfig(enabled=True),
                              CUDAGraphConfig(enabled=False, capture_sizes=[T]), extra)
@@ -370,7 +385,8 @@ def decode_config(torch, steps, warmup, layers=32):
     for name, knobs, graphs in (("serialized_eager", {"serialize": True}, False), ("overlapped_eager", {}, False),
                                 ("overlapped_sub_graph_replay", {}, True),
                                 ("stream_per_nano_batch_sub_graph_replay", {"streams": "by_nano_batch"}, True)):
-        extra = {"min_nano_split_tokens": 1, "dump_graph": False, "max_tokens": seqs, "fuse_silu_epilogue": True}
+        extra = {"min_nano_split_tokens": 1, "dump_graph": False, "max_tokens": seqs, "fuse_silu_epilogue": True,
+                 **EXTRA_KNOBS}
         extra.update(knobs)
         cfg = DynaFlowConfig("dynaflow_amd.schedulers:DecoderOverlapScheduler", 2, InductorConfig(enabled=True),
                              CUDAGraphConfig(enabled=graphs, capture_sizes=[half, seqs]), extra)
@@ -463,6 +479,7 @@ def cpu_baseline(torch):
 
 def main() -> int:
     args = parse_args()
+    read_knobs(args.knob)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported in this build "
               "(the path has no multi-GPU part)", file=sys.stderr)
