@@ -41,6 +41,8 @@ class StaggeredScheduler(OpSchedulerBase):
         self.stream_policy: str = config.knob("streams", "by_kind")
         if self.stream_policy not in ("by_kind", "by_nano_batch"):
             raise ValueError(f"unknown stream policy {self.stream_policy!r}")
+        # "staggered": nano-batch 0 starts one sub-graph ahead; "round_robin": all nano-batches in step
+        self.order: str = config.knob("schedule", "staggered")
 
     def get_split_rules(self) -> list[MatchingRule]:
         return self._split_rules
@@ -63,7 +65,7 @@ class StaggeredScheduler(OpSchedulerBase):
     async def schedule(self, context: ExecutionContext) -> None:
         lanes = context.split_config.num_nano_batches
         live = list(range(lanes))
-        if lanes >= 2:
+        if lanes >= 2 and self.order != "round_robin":
             head = await context.pop(0)
             if head is None:
                 live.remove(0)
