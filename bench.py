@@ -255,7 +255,10 @@ def fp8_config(torch, steps, warmup):
     layer = Fp8SwiGLU.from_weights(*parts)
     del parts
     results = {}
-    for name, knobs in (("serialized", {"serialize": True}), ("overlapped", {"whole_graph": True})):
+    for name, knobs in (("serialized", {"serialize": True}), ("overlapped", {"whole_graph": True}),
+                        ("overlapped_fused_gate_up", {"whole_graph": True, "fuse_silu_epilogue": True})):
+        # the fused mode: gate, up and SiLU*mul + absmax in ONE GEMM launch, cut in front of the down projection
+        layer.fuse_gate_up = bool(knobs.get("fuse_silu_epilogue", False))
         extra = {"min_nano_split_tokens": 64, "num_nano_batches": splits, "dump_graph": False, **EXTRA_KNOBS}
         extra.update(knobs)
         cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", splits, InductorConfig(enabled=True),
@@ -283,14 +286,15 @@ def fp8_config(torch, steps, warmup):
                 torch.cuda.synchronize()
                 results[f"{name}_{mode}_ms"] = (time.perf_counter() - t0) * 1e3 / steps
     flops = 6.0 * tokens * hidden * inter
-    best = results["overlapped_graph_ms"]
+    best = min(results["overlapped_graph_ms"], results["overlapped_fused_gate_up_graph_ms"])
     return {
         "metric": "fp8 MLP-layer tokens/s, 70B-shape e4m3, 1 MI355X",
         "value": tokens / (best * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": best, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3",
         "data": "synthetic",
         "config": {"workload": "fp8 70B-shaped SwiGLU MLP layer, x[8192,8192], I=28672, 4 nano-batches of 2048, "
-                               "per-tensor activation / per-channel weight scales, bf16 output"},
+                               "per-tensor activation / per-channel weight scales, bf16 output; the best of "
+                               "the separate gate / up / SiLU*mul launches and the one-launch form is reported"},
         "timings": results,
         "layer": {"tflops": flops / (best * 1e-3) / 1e12, "frac_of_fp8_mfma_peak": flops / (best * 1e-3) / 1e12 / 5000.0},
         "overlap_speedup": results["serialized_eager_ms"] / best,

@@ -73,6 +73,8 @@ SIGNATURES: dict[str, tuple] = {
         c_int,
         [_P, c_int64, _P, c_int64, _P, c_int64, _P, _P, c_int, c_int, c_int, c_int, _P],
     ),
+    "dfhip_gemm_fp8_gate_up_silu_absmax": (c_int, [_P, c_int64, _P, _P, c_int64, _P, c_int64, _P, _P, _P, _P, c_int,
+                                                     c_int, c_int, _P]),
     "dfhip_silu_mul_bf16": (c_int, [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P]),
     "dfhip_silu_mul_f32": (c_int, [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, _P]),
     "dfhip_rmsnorm_bf16": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, c_float, _P]),

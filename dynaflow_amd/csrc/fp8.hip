@@ -242,14 +242,21 @@ gemm_fp8_nt_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W,
 constexpr int F8_UNIT = 32768, F8_NUNITS = 5, F8_RING_LDS = F8_UNIT * F8_NUNITS;
 constexpr int F8_GROUP_M = 4, F8_EROW = 272;
 
+// FUSED: the W half of a slab holds 128 rows of W (gate) and the matching 128 rows of W2 (up); the tile
+// then is 256 x 128 outputs, N counts those, and the epilogue writes act = bf16(silu(bf16 g) * bf16 u) -
+// the roundings of the separate GEMMs and of silu_mul_absmax_kernel, so the same bits - and folds
+// max |act| into amax[0].
+template <bool FUSED>
 __global__ void __launch_bounds__(256)
-gemm_fp8_ring_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, uint16_t* __restrict__ C,
-                     const float* __restrict__ a_scale, const float* __restrict__ w_scale, int M, int N, int K,
-                     int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n) {
+gemm_fp8_ring_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ W, const uint8_t* __restrict__ W2,
+                     uint16_t* __restrict__ C, const float* __restrict__ a_scale, const float* __restrict__ w_scale,
+                     const float* __restrict__ w2_scale, float* __restrict__ amax, int M, int N, int K, int64_t lda,
+                     int64_t ldw, int64_t ldc, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave & 1, wave_n = wave >> 1;
+  constexpr int TILE_N = FUSED ? 128 : 256;    // output columns of a tile
 
   const int tile = remap_xcd(blockIdx.x, tiles_m * tiles_n);
   const int per_panel = F8_GROUP_M * tiles_n;
@@ -257,7 +264,7 @@ gemm_fp8_ring_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ 
   const int rows_in_panel = (tiles_m - first_m) < F8_GROUP_M ? (tiles_m - first_m) : F8_GROUP_M;
   const int in_panel = tile % per_panel;
   const int m0 = (first_m + in_panel % rows_in_panel) * 256;
-  const int n0 = (in_panel / rows_in_panel) * 256;
+  const int n0 = (in_panel / rows_in_panel) * TILE_N;
   const int KT = K / FBK;
 
   const uint8_t* a_src[8];
@@ -267,9 +274,14 @@ gemm_fp8_ring_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ 
     const int row = (wave * 8 + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     int ar = m0 + row; ar = ar < M ? ar : M - 1;
-    int wr = n0 + row; wr = wr < N ? wr : N - 1;
     a_src[t] = A + (int64_t)ar * lda + chunk * 16;
-    w_src[t] = W + (int64_t)wr * ldw + chunk * 16;
+    if (FUSED) {
+      int wr = n0 + (row & 127); wr = wr < N ? wr : N - 1;
+      w_src[t] = (row < 128 ? W : W2) + (int64_t)wr * ldw + chunk * 16;
+    } else {
+      int wr = n0 + row; wr = wr < N ? wr : N - 1;
+      w_src[t] = W + (int64_t)wr * ldw + chunk * 16;
+    }
   }
   const uint32_t wave_lds = wave * 8 * 1024;
   auto dma_a = [&](int t, int slab, int unit) {
@@ -366,9 +378,9 @@ gemm_fp8_ring_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ 
   for (int j = 0; j < 4; ++j)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      int n = n0 + wave_n * 128 + j * 32 + g * 8 + fhalf * 4;
+      int n = n0 + (FUSED ? 0 : wave_n * 128) + j * 32 + g * 8 + fhalf * 4;
       n = n < N ? n : N - 4;   // columns past the edge are never stored; keep the scale load in bounds
-      const f32x4 ws = *reinterpret_cast<const f32x4*>(w_scale + n);
+      const f32x4 ws = *reinterpret_cast<const f32x4*>((FUSED && wave_n ? w2_scale : w_scale) + n);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         u32x2 v;
@@ -378,6 +390,41 @@ gemm_fp8_ring_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ 
       }
     }
   DFHIP_PIN;
+  if (FUSED) {
+    // gate blocks sit in the parks of waves 0, 1 (rows 0..127, 128..255), up blocks in those of waves 2, 3;
+    // wave w combines rows (w & 1) * 128 + (w >> 1) * 64 .. + 64 of the tile
+    __syncthreads();
+    const uint8_t* gpark = smem + (wave & 1) * (128 * F8_EROW);
+    const uint8_t* upark = smem + ((wave & 1) + 2) * (128 * F8_EROW);
+    const int row0 = (wave >> 1) * 64;
+    float vmax = 0.0f;
+#pragma unroll 4
+    for (int p = 0; p < 16; ++p) {
+      const int id = p * 64 + lane;
+      const int row = row0 + (id >> 4), c = id & 15;
+      const u32x4 gv = *reinterpret_cast<const u32x4*>(gpark + row * F8_EROW + c * 16);
+      const u32x4 uv = *reinterpret_cast<const u32x4*>(upark + row * F8_EROW + c * 16);
+      u32x4 o;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float lo = silu_f32(bf16_bits_to_f32(gv[w] & 0xffffu)) * bf16_bits_to_f32(uv[w] & 0xffffu);
+        const float hi = silu_f32(__uint_as_float(gv[w] & 0xffff0000u)) * __uint_as_float(uv[w] & 0xffff0000u);
+        o[w] = pack2_bf16(lo, hi);
+      }
+      const int m = m0 + (wave & 1) * 128 + row, n = n0 + c * 8;
+      if (m < M && n < N) {
+        *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = o;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          vmax = fmaxf(vmax, fabsf(bf16_bits_to_f32(o[w] & 0xffffu)));
+          vmax = fmaxf(vmax, fabsf(__uint_as_float(o[w] & 0xffff0000u)));
+        }
+      }
+    }
+    vmax = wave_max(vmax);
+    if (lane == 0) atomic_max_nonneg(amax, vmax);
+    return;
+  }
   const int m_base = m0 + wave_m * 128, n_base = n0 + wave_n * 128;
 #pragma unroll 4
   for (int p = 0; p < 32; ++p) {
@@ -393,15 +440,34 @@ int launch_fp8_ring(const void* A, int64_t lda, const void* W, int64_t ldw, void
                     const float* a_scale, const float* w_scale, int M, int N, int K, hipStream_t stream) {
   static bool lds_opted_in = false;
   if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fp8_ring_kernel),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fp8_ring_kernel<false>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, F8_RING_LDS) != hipSuccess)
       return DFHIP_ERR_LAUNCH;
     lds_opted_in = true;
   }
   const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
-  hipLaunchKernelGGL(gemm_fp8_ring_kernel, dim3(tiles_m * tiles_n), dim3(256), F8_RING_LDS, stream,
-                     static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(W), static_cast<uint16_t*>(C),
-                     a_scale, w_scale, M, N, K, lda, ldw, ldc, tiles_m, tiles_n);
+  hipLaunchKernelGGL(gemm_fp8_ring_kernel<false>, dim3(tiles_m * tiles_n), dim3(256), F8_RING_LDS, stream,
+                     static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(W), nullptr,
+                     static_cast<uint16_t*>(C), a_scale, w_scale, nullptr, nullptr, M, N, K, lda, ldw, ldc, tiles_m,
+                     tiles_n);
+  return dfhip_check_launch();
+}
+
+int launch_fp8_ring_fused(const void* A, int64_t lda, const void* Wg, const void* Wu, int64_t ldw, void* act,
+                          int64_t ld_act, const float* a_scale, const float* wg_scale, const float* wu_scale,
+                          float* amax, int M, int I, int K, hipStream_t stream) {
+  static bool lds_opted_in = false;
+  if (!lds_opted_in) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fp8_ring_kernel<true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, F8_RING_LDS) != hipSuccess)
+      return DFHIP_ERR_LAUNCH;
+    lds_opted_in = true;
+  }
+  const int tiles_m = (M + 255) / 256, tiles_n = (I + 127) / 128;
+  hipLaunchKernelGGL(gemm_fp8_ring_kernel<true>, dim3(tiles_m * tiles_n), dim3(256), F8_RING_LDS, stream,
+                     static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(Wg), static_cast<const uint8_t*>(Wu),
+                     static_cast<uint16_t*>(act), a_scale, wg_scale, wu_scale, amax, M, I, K, lda, ldw, ld_act,
+                     tiles_m, tiles_n);
   return dfhip_check_launch();
 }
 
@@ -688,6 +754,22 @@ extern "C" int dfhip_gemm_fp8_nt_variant(const void* A, int64_t lda, const void*
     case 2: return launch_fp8_ring224(A, lda, W, ldw, C, ldc, a_scale, w_scale, M, N, K, s);
     default: return DFHIP_ERR_BAD_ARGUMENT;
   }
+}
+
+extern "C" int dfhip_gemm_fp8_gate_up_silu_absmax(const void* A, int64_t lda, const void* W_gate, const void* W_up,
+                                                  int64_t ldw, void* act, int64_t ld_act, const float* a_scale,
+                                                  const float* w_gate_scale, const float* w_up_scale, float* amax,
+                                                  int M, int I, int K, dfhip_stream_t stream) {
+  if (!A || !W_gate || !W_up || !act || !a_scale || !w_gate_scale || !w_up_scale || !amax)
+    return DFHIP_ERR_NULL_POINTER;
+  if (M < 1 || I < 8 || K < 1 || K % FBK != 0 || I % 8 != 0) return DFHIP_ERR_BAD_SHAPE;
+  if (lda < K || ldw < K || ld_act < I) return DFHIP_ERR_BAD_STRIDE;
+  if (lda % 16 || ldw % 16 || ld_act % 8 || !dfhip_aligned16(A) || !dfhip_aligned16(W_gate) ||
+      !dfhip_aligned16(W_up) || !dfhip_aligned16(act) || !dfhip_aligned16(w_gate_scale) ||
+      !dfhip_aligned16(w_up_scale))
+    return DFHIP_ERR_BAD_ALIGNMENT;
+  return launch_fp8_ring_fused(A, lda, W_gate, W_up, ldw, act, ld_act, a_scale, w_gate_scale, w_up_scale, amax, M, I,
+                               K, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int dfhip_gemm_fp8_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,

@@ -51,6 +51,10 @@ _lib.define("silu_mul_quant_fp8(Tensor gate, Tensor up) -> (Tensor, Tensor)")
 _lib.define("linear_fp8(Tensor x_q, Tensor w_q, Tensor x_scale, Tensor w_scale) -> Tensor")
 _lib.define("linear_fp8_variant(Tensor x_q, Tensor w_q, Tensor x_scale, Tensor w_scale, int variant) -> Tensor")
 _lib.define("linear_fp8_to_output(Tensor x_q, Tensor w_q, Tensor x_scale, Tensor w_scale) -> Tensor")
+_lib.define(
+    "gate_up_silu_quant_fp8(Tensor x_q, Tensor w_gate_q, Tensor w_up_q, Tensor x_scale, Tensor w_gate_scale, "
+    "Tensor w_up_scale) -> (Tensor, Tensor)"
+)
 
 FP8_DTYPE = torch.float8_e4m3fn
 FP8_MAX = 448.0
@@ -562,6 +566,41 @@ def _silu_mul_quant_fp8_impl(gate: torch.Tensor, up: torch.Tensor):
     return q.view(gate.shape), scale
 
 
+def _gate_up_silu_quant_fp8_impl(x_q, w_gate_q, w_up_q, x_scale, w_gate_scale, w_up_scale):
+    """The fp8 gate and up projections with SiLU*mul as the GEMM's epilogue, then the re-quantisation:
+    returns what ``silu_mul_quant_fp8(linear_fp8(x, w_gate), linear_fp8(x, w_up))`` returns, bit for bit."""
+    _require_device(x_q, w_gate_q, w_up_q, x_scale, w_gate_scale, w_up_scale)
+    lib = _cabi.load()
+    if x_q.dtype != FP8_DTYPE or w_gate_q.dtype != FP8_DTYPE or w_up_q.dtype != FP8_DTYPE:
+        raise RuntimeError("gate_up_silu_quant_fp8: e4m3fn operands only")
+    if any(t.dtype != torch.float32 for t in (x_scale, w_gate_scale, w_up_scale)):
+        raise RuntimeError("gate_up_silu_quant_fp8: fp32 scales only")
+    a, M, K, lda = _rows(x_q)
+    wg, I, Kw, ldg = _rows(w_gate_q)
+    wu, Iu, Ku, ldu = _rows(w_up_q)
+    if K != Kw or K != Ku or I != Iu or w_gate_scale.numel() != I or w_up_scale.numel() != I or x_scale.numel() != 1:
+        raise RuntimeError("gate_up_silu_quant_fp8: shape mismatch")
+    if ldg != ldu:
+        wg, wu = wg.contiguous(), wu.contiguous()
+        ldg = K
+    act = torch.empty((M, I), dtype=torch.bfloat16, device=x_q.device)
+    amax = torch.empty(1, dtype=torch.float32, device=x_q.device)
+    scale = torch.empty(1, dtype=torch.float32, device=x_q.device)
+    q = torch.empty((M, I), dtype=FP8_DTYPE, device=x_q.device)
+    if M > 0:
+        _fill_zero(amax)
+        rc = lib.dfhip_gemm_fp8_gate_up_silu_absmax(
+            a.data_ptr(), lda, wg.data_ptr(), wu.data_ptr(), ldg, act.data_ptr(), I, x_scale.data_ptr(),
+            w_gate_scale.contiguous().data_ptr(), w_up_scale.contiguous().data_ptr(), amax.data_ptr(), M, I, K,
+            _stream(),
+        )
+        _cabi.check("dfhip_gemm_fp8_gate_up_silu_absmax", rc)
+        rc = lib.dfhip_quant_fp8_bf16(act.data_ptr(), I, q.data_ptr(), I, M, I, amax.data_ptr(), scale.data_ptr(),
+                                      _stream())
+        _cabi.check("dfhip_quant_fp8_bf16", rc)
+    return q.view(*x_q.shape[:-1], I), scale
+
+
 def _linear_fp8_impl(x_q, w_q, x_scale, w_scale, variant: int = -1, to_output: bool = False):
     _require_device(x_q, w_q, x_scale, w_scale)
     lib = _cabi.load()
@@ -585,6 +624,13 @@ def _linear_fp8_impl(x_q, w_q, x_scale, w_scale, variant: int = -1, to_output: b
 
 _lib.impl("quant_fp8", _quant_fp8_impl, "CUDA")
 _lib.impl("silu_mul_quant_fp8", _silu_mul_quant_fp8_impl, "CUDA")
+_lib.impl("gate_up_silu_quant_fp8", _gate_up_silu_quant_fp8_impl, "CUDA")
+torch.library.register_fake(
+    "dynaflow_hip::gate_up_silu_quant_fp8",
+    lambda x_q, wg, wu, xs, wgs, wus: (x_q.new_empty((*x_q.shape[:-1], wg.shape[0]), dtype=FP8_DTYPE),
+                                       x_q.new_empty((1,), dtype=torch.float32)),
+    lib=_lib,
+)
 _lib.impl("linear_fp8", lambda x_q, w_q, xs, ws: _linear_fp8_impl(x_q, w_q, xs, ws), "CUDA")
 _lib.impl("linear_fp8_variant", lambda x_q, w_q, xs, ws, v: _linear_fp8_impl(x_q, w_q, xs, ws, v), "CUDA")
 _lib.impl("linear_fp8_to_output", lambda x_q, w_q, xs, ws: _linear_fp8_impl(x_q, w_q, xs, ws, to_output=True), "CUDA")
@@ -632,3 +678,4 @@ silu_mul_quant_fp8 = torch.ops.dynaflow_hip.silu_mul_quant_fp8
 linear_fp8 = torch.ops.dynaflow_hip.linear_fp8
 linear_fp8_variant = torch.ops.dynaflow_hip.linear_fp8_variant
 linear_fp8_to_output = torch.ops.dynaflow_hip.linear_fp8_to_output
+gate_up_silu_quant_fp8 = torch.ops.dynaflow_hip.gate_up_silu_quant_fp8

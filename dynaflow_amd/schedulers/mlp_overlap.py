@@ -55,19 +55,25 @@ def _follows_product(node_list, start_idx: int) -> bool:
     node = node_list[start_idx]
     producer = node.args[0] if node.args else None
     name = getattr(getattr(producer, "target", None), "__name__", "")
-    return getattr(producer, "op", None) == "call_function" and name.split(".")[0] in ("mul", "silu_mul", "gate_up_silu")
+    if name == "getitem" and getattr(producer, "args", None):     # first output of an operator with two
+        producer = producer.args[0]
+        name = getattr(getattr(producer, "target", None), "__name__", "")
+    return getattr(producer, "op", None) == "call_function" and name.split(".")[0] in (
+        "mul", "silu_mul", "gate_up_silu", "gate_up_silu_quant_fp8")
 
 
 def mlp_split_rules_fused() -> list[MatchingRule]:
     """Cut only in front of the down projection: {gate, up, silu, mul} | {down}, so that the
     SiLU*mul can become the epilogue of the gate/up GEMM."""
-    return [MatchingRule(condition=Op(_LINEAR), hook=_follows_product)]
+    return [MatchingRule(condition=Op(_LINEAR), hook=_follows_product),
+            MatchingRule(condition=Op(r"linear_fp8(\.default)?"), hook=_follows_product)]
 
 
 def mlp_tag_rules_fused() -> dict[MatchingRule, set[str]]:
     # inside the down-projection sub-graph the product is just an input, so the sub-graph that
     # holds the product is the one that gets a tag (and the second stream)
-    return {MatchingRule(condition=Op(_MUL)): {HEAD_TAG}}
+    return {MatchingRule(condition=Op(_MUL)): {HEAD_TAG},
+            MatchingRule(condition=Op(r"gate_up_silu_quant_fp8(\.default)?")): {HEAD_TAG}}
 
 
 def mlp_tag_rules() -> dict[MatchingRule, set[str]]:

@@ -151,6 +151,18 @@ int dfhip_gemm_fp8_nt(const void* A, int64_t lda, const void* W, int64_t ldw, vo
 int dfhip_gemm_fp8_nt_variant(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
                               const float* a_scale, const float* w_scale, int M, int N, int K, int variant,
                               dfhip_stream_t stream);
+/* Gate and up projection of the fp8 MLP block with the SiLU*mul as the epilogue of ONE launch:
+ *   g = bf16(a_scale * wg_scale[i] * A W_gate^T), u likewise with W_up,
+ *   act[m,i] = bf16( silu(g) * u ),   amax[0] = max(amax[0], max |act|)
+ * - the roundings of two dfhip_gemm_fp8_nt launches followed by dfhip_silu_mul_absmax_bf16, so the
+ * same bits.  amax must hold 0 (or an earlier maximum) before the call; dfhip_quant_fp8_bf16 then
+ * re-quantises act.  W_gate and W_up: [I, K] e4m3fn with one row stride.  In the reference these are
+ * the FX nodes linear, linear, silu, mul of the host model's MLP (engine.py:381 runs them through
+ * PyTorch); the wave-specialised fused kernel of examples/ae/OVERLAP.md:8-12 is the same idea. */
+int dfhip_gemm_fp8_gate_up_silu_absmax(const void* A, int64_t lda, const void* W_gate, const void* W_up,
+                                       int64_t ldw, void* act, int64_t ld_act, const float* a_scale,
+                                       const float* w_gate_scale, const float* w_up_scale, float* amax, int M,
+                                       int I, int K, dfhip_stream_t stream);
 
 /* ------------------------------------------------------------ elementwise
  *

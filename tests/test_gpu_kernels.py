@@ -407,3 +407,27 @@ def test_gemm_fp8_variants_agree(ops, M, N, K, variant):
     want = mlp.dequant(xq, xs) @ mlp.dequant(wq, ws).t()
     assert got.shape == (M, N) and rel_err(got.float(), want) < 2 ** -7
     assert torch.equal(got, ops.linear_fp8_variant(*args, 1))
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 8, 128), (300, 264, 384), (512, 1024, 1024), (2048, 3584, 256), (1100, 2056, 384)])
+def test_fp8_gate_up_silu_epilogue_has_the_bits_of_the_separate_operators(ops, M, I, K):
+    """One launch for the gate and up projection with SiLU*mul + absmax as the epilogue, then the re-quantiser:
+    codes and scale must equal ``silu_mul_quant_fp8(linear_fp8(x, w_gate), linear_fp8(x, w_up))`` bit for bit
+    (ragged last row / column tiles included), run to run as well."""
+    x = randn((M, K), 30).bfloat16()
+    wg = randn((I, K), 31, 0.05).bfloat16()
+    wu = randn((I, K), 32, 0.05).bfloat16()
+    xq, xs = mlp.quant_e4m3(x)
+    wgq, wgs = mlp.quant_e4m3_per_channel(wg)
+    wuq, wus = mlp.quant_e4m3_per_channel(wu)
+    f8 = torch.float8_e4m3fn
+    xq, wgq, wuq = xq.cuda().view(f8), wgq.cuda().view(f8), wuq.cuda().view(f8)
+    xs, wgs, wus = xs.cuda(), wgs.cuda(), wus.cuda()
+    want_q, want_s = ops.silu_mul_quant_fp8(ops.linear_fp8(xq, wgq, xs, wgs), ops.linear_fp8(xq, wuq, xs, wus))
+    got_q, got_s = ops.gate_up_silu_quant_fp8(xq, wgq, wuq, xs, wgs, wus)
+    torch.cuda.synchronize()
+    assert got_q.shape == (M, I) and got_q.dtype == f8
+    assert torch.equal(got_s, want_s)
+    assert torch.equal(got_q.view(torch.uint8), want_q.view(torch.uint8))
+    again_q, again_s = ops.gate_up_silu_quant_fp8(xq, wgq, wuq, xs, wgs, wus)
+    assert torch.equal(again_q.view(torch.uint8), got_q.view(torch.uint8)) and torch.equal(again_s, got_s)

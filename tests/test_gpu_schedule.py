@@ -162,7 +162,7 @@ def test_whole_schedule_graph_replay():
     assert torch.equal(y, want)
 
 
-def fp8_layer(tokens, hidden, inter):
+def fp8_layer(tokens, hidden, inter, fuse_gate_up=False):
     from dynaflow_amd.fp8_mlp import Fp8SwiGLU
 
     x, wg, wu, wd = mlp.make_inputs(tokens, hidden, inter, torch.bfloat16)
@@ -170,7 +170,7 @@ def fp8_layer(tokens, hidden, inter):
     buffers = []
     for codes, scale in quantised:
         buffers += [codes.cuda().view(torch.float8_e4m3fn), scale.cuda()]
-    return Fp8SwiGLU(*buffers), x, quantised, (wg, wu, wd)
+    return Fp8SwiGLU(*buffers, fuse_gate_up=fuse_gate_up), x, quantised, (wg, wu, wd)
 
 
 def test_fp8_layer_against_dequantised_reference():
@@ -218,6 +218,45 @@ def test_fp8_layer_through_the_manager_with_four_nano_batches():
     want = mlp.mlp_fp8_dequant_reference(x, wg_q, wg_s, wu_q, wu_s, wd_q, wd_s, split.split_indices)
     assert rel_err(y.float(), want.float()) < TOL["fp8"]
     assert torch.equal(y, layer.forward_schedule(xg, split.split_indices))
+
+
+def test_fp8_layer_with_fused_gate_up_epilogue_through_the_manager():
+    """The fp8 block with gate/up/SiLU*mul as one operator, cut in front of the down projection: the fused
+    sub-graph of one nano-batch beside the down projection of the previous one; same bits as the unfused block."""
+    from dynaflow_amd import ops
+    from dynaflow_amd.backend import make_backend
+    from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
+    from dynaflow_amd.manager import DynaFlowManager
+
+    tokens = 512
+    layer, x, quantised, _ = fp8_layer(tokens, 1024, 2048, fuse_gate_up=True)
+    plain, *_ = fp8_layer(tokens, 1024, 2048)
+    cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", 4, InductorConfig(enabled=True),
+                         CUDAGraphConfig(enabled=False, capture_sizes=[tokens]),
+                         {"min_nano_split_tokens": 1, "num_nano_batches": 4, "dump_graph": False,
+                          "fuse_silu_epilogue": True})
+    manager = DynaFlowManager()
+    torch._dynamo.reset()
+    xg = x.cuda()
+    torch._dynamo.mark_dynamic(xg, 0)
+    compiled = torch.compile(layer, backend=make_backend(manager, cfg), fullgraph=True)
+    with torch.no_grad():
+        manager.prepare(tokens, [tokens])
+        compiled(xg)
+        split = manager.prepare(tokens, [tokens])
+        y = compiled(xg)
+    torch.cuda.synchronize()
+    names = [n.target for n in manager.graph_module.graph.nodes if n.op == "call_module"]
+    assert len(names) == 2
+    head = [n.target for n in manager.graph_module.__dict__[names[0]].callable_dynamic.graph.nodes
+            if n.op == "call_function"]
+    assert any(getattr(t, "overloadpacket", t) is ops.gate_up_silu_quant_fp8 for t in head)
+    assert getattr(manager.graph_module, names[0]).tag == {"head"}
+    assert split.split_indices == [0, 128, 256, 384, 512]
+    (wg_q, wg_s), (wu_q, wu_s), (wd_q, wd_s) = quantised
+    want = mlp.mlp_fp8_dequant_reference(x, wg_q, wg_s, wu_q, wu_s, wd_q, wd_s, split.split_indices)
+    assert rel_err(y.float(), want.float()) < TOL["fp8"]
+    assert torch.equal(y, plain.forward_schedule(xg, split.split_indices))
 
 
 def test_piecewise_graphs_capture_in_dryrun_and_replay():
