@@ -14,6 +14,8 @@ it deep-copies the sub-``GraphModule`` and replaces
 * ``add(r, linear(x, w))`` (bf16, same shapes, the linear used once) -> ``dynaflow_hip.linear_add``
   (the residual addition as the GEMM's epilogue; same roundings, same bits)
 
+* two or more bf16 ``linear`` nodes of the same activation (q / k / v projections) -> ONE
+  ``dynaflow_hip.linear_multi`` against the stacked weights, results as column ranges of one buffer
 * the ``linear`` / ``linear_add`` whose result is what the sub-graph returns -> ``*_to_output``
   (writes into rows offered by the engine, so the nano-batch outputs need no concatenation)
 
@@ -276,6 +278,29 @@ def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False) -> tuple[
             stats["gate_up_silu"] += 1
             stats["linear"] -= 2
             stats["silu_mul"] -= 1
+
+    # Several bf16 projections of one activation (q / k / v; gate / up when they are not fused with the product)
+    # become one GEMM against the stacked weights: narrow products (1024 columns) fill the chip badly on their own.
+    groups: dict[fx.Node, list[fx.Node]] = {}
+    for node in graph.nodes:
+        if node.op == "call_function" and node.target is ops.linear and isinstance(node.args[0], fx.Node):
+            ex, ew = _example(node.args[0]), _example(node.args[1])
+            if (isinstance(ex, torch.Tensor) and ex.dtype == torch.bfloat16 and isinstance(ew, torch.Tensor)
+                    and isinstance(node.args[1], fx.Node) and node.args[1].op == "placeholder"
+                    and _static_int(ew.shape[0]) is not None and _static_int(ew.shape[0]) % 8 == 0):
+                groups.setdefault(node.args[0], []).append(node)
+    for x, members in groups.items():
+        if len(members) < 2:
+            continue
+        with graph.inserting_before(members[0]):
+            multi = graph.call_function(ops.linear_multi, (x, [m.args[1] for m in members]))
+            parts = [graph.call_function(operator.getitem, (multi, i)) for i in range(len(members))]
+        for member, part in zip(members, parts):
+            part.meta = dict(member.meta)
+            member.replace_all_uses_with(part)
+            graph.erase_node(member)
+        stats["linear_multi"] = stats.get("linear_multi", 0) + 1
+        stats["linear"] -= len(members)
 
     # The projection whose result the sub-graph returns (and nothing else reads) may write straight into the
     # rows that the engine offers for the model output; without an offer it behaves like the plain operator.

@@ -41,6 +41,7 @@ _lib.define("rope(Tensor t, Tensor cos, Tensor sin) -> Tensor")
 _lib.define("causal_attention(Tensor q, Tensor k, Tensor v) -> Tensor")
 _lib.define("linear_add(Tensor x, Tensor weight, Tensor residual) -> Tensor")
 _lib.define("linear_to_output(Tensor x, Tensor weight) -> Tensor")
+_lib.define("linear_multi(Tensor x, Tensor[] weights) -> Tensor[]")
 _lib.define("linear_add_to_output(Tensor x, Tensor weight, Tensor residual) -> Tensor")
 _lib.define(
     "decode_attention(Tensor qkv, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor slots, Tensor lengths, "
@@ -230,6 +231,41 @@ torch.library.register_fake("dynaflow_hip::linear_to_output", _linear_fake, lib=
 torch.library.register_fake("dynaflow_hip::linear_variant", lambda x, w, v: _linear_fake(x, w), lib=_lib)
 
 
+# ------------------------------------------- several projections of one activation
+#: row-wise concatenations of weight groups, keyed by the members' storage and version counters (a weight that
+#: is written to gets a new entry; entries are never dropped, which suits frozen inference weights)
+_stacked_weights: dict[tuple, torch.Tensor] = {}
+
+
+def _linear_multi_impl(x: torch.Tensor, weights: list[torch.Tensor]) -> list[torch.Tensor]:
+    """``[x @ w.T for w in weights]`` as ONE GEMM against the row-wise concatenation of the weights (made on the
+    first call and kept); the results are column ranges of one buffer.  q, k and v projections of 4096 + 1024 +
+    1024 columns fill the rounds of 256 workgroups as one 6144-column product, not as three."""
+    _require_device(x, *weights)
+    if x.dtype != torch.bfloat16 or any(w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != x.shape[-1]
+                                         or w.shape[0] % 8 for w in weights):
+        raise RuntimeError("linear_multi: bf16 activation and [N_i, K] bf16 weights with N_i % 8 == 0 expected")
+    key = tuple((w.data_ptr(), w._version, w.shape[0]) for w in weights)
+    stacked = _stacked_weights.get(key)
+    if stacked is None:
+        if torch.cuda.is_current_stream_capturing():
+            return [_linear_impl(x, w) for w in weights]      # no allocation that outlives the capture
+        stacked = torch.cat([w.detach() for w in weights], dim=0).contiguous()
+        _stacked_weights[key] = stacked
+    out = _linear_impl(x, stacked)
+    parts, first = [], 0
+    for w in weights:
+        parts.append(out[..., first:first + w.shape[0]])
+        first += w.shape[0]
+    return parts
+
+
+_lib.impl("linear_multi", _linear_multi_impl, "CUDA")
+torch.library.register_fake(
+    "dynaflow_hip::linear_multi", lambda x, weights: [_linear_fake(x, w) for w in weights], lib=_lib
+)
+
+
 # ------------------------------------------------ projection + residual addition
 def _linear_add_impl(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor,
                      to_output: bool = False) -> torch.Tensor:
@@ -376,6 +412,15 @@ torch.library.register_fake(
 )
 
 
+def _token_rows(t: torch.Tensor, what: str):
+    """[B, S, H, d] with contiguous heads -> (tensor, token stride in elements); a copy only if the tokens
+    are not evenly strided rows (a column range of a wider [tokens, columns] buffer is used in place)."""
+    if (t.dim() != 4 or t.stride(3) != 1 or t.stride(2) != t.shape[3] or t.stride(1) < t.shape[2] * t.shape[3]
+            or t.stride(0) != t.shape[1] * t.stride(1)):
+        t = t.contiguous()
+    return t, t.stride(1)
+
+
 # ------------------------------------------------------------------ rope
 def _rope_impl(t: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
     """t [B, S, heads, d] bf16 (contiguous), cos/sin [S, d/2] fp32 -> rotated tensor of the same shape."""
@@ -386,11 +431,11 @@ def _rope_impl(t: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
     B, S, heads, d = t.shape
     if cos.shape != (S, d // 2) or sin.shape != (S, d // 2):
         raise RuntimeError("rope: table shape mismatch")
-    src = t.contiguous()
-    out = torch.empty_like(src)
+    src, ld_src = _token_rows(t, "t")            # a column range of a wider buffer is read in place
+    out = torch.empty((B, S, heads, d), dtype=t.dtype, device=t.device)
     if src.numel() > 0:
         rc = lib.dfhip_rope_bf16(
-            src.data_ptr(), heads * d, out.data_ptr(), heads * d, cos.contiguous().data_ptr(),
+            src.data_ptr(), ld_src, out.data_ptr(), heads * d, cos.contiguous().data_ptr(),
             sin.contiguous().data_ptr(), B * S, heads, d, S, _stream(),
         )
         _cabi.check("dfhip_rope_bf16", rc)
@@ -402,13 +447,6 @@ torch.library.register_fake("dynaflow_hip::rope", lambda t, cos, sin: torch.empt
 
 
 # ------------------------------------------------------ prefill attention
-def _token_rows(t: torch.Tensor, what: str):
-    """[B, S, H, 128] with contiguous heads -> (tensor, token stride in elements)."""
-    if t.dim() != 4 or t.shape[3] != 128 or t.stride(3) != 1 or t.stride(2) != 128 or t.stride(0) != t.shape[1] * t.stride(1):
-        t = t.contiguous()
-    return t, t.stride(1)
-
-
 def _causal_attention_impl(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
     """q [B, S, Hq, 128], k / v [B, S, Hkv, 128] (bf16) -> softmax(q k^T / sqrt(128), causal) v as [B, S, Hq, 128]."""
     _require_device(q, k, v)
@@ -672,6 +710,7 @@ decode_attention = torch.ops.dynaflow_hip.decode_attention
 causal_attention = torch.ops.dynaflow_hip.causal_attention
 linear_add = torch.ops.dynaflow_hip.linear_add
 linear_to_output = torch.ops.dynaflow_hip.linear_to_output
+linear_multi = torch.ops.dynaflow_hip.linear_multi
 linear_add_to_output = torch.ops.dynaflow_hip.linear_add_to_output
 quant_fp8 = torch.ops.dynaflow_hip.quant_fp8
 silu_mul_quant_fp8 = torch.ops.dynaflow_hip.silu_mul_quant_fp8

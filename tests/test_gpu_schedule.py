@@ -57,7 +57,9 @@ def test_subgraphs_run_on_hip_operators():
     for name in ("submod_0", "submod_1"):
         backend = manager.graph_module.__dict__[name]
         targets = [n.target for n in backend.callable_dynamic.graph.nodes if n.op == "call_function"]
-        assert all(t in (ops.linear, ops.linear_to_output, ops.silu_mul) for t in targets), targets
+        import operator
+
+        assert all(t in (ops.linear, ops.linear_to_output, ops.silu_mul, operator.getitem) for t in targets), targets
 
 
 def test_config1_fp32_matches_cpu_reference_path():
@@ -430,12 +432,13 @@ def test_decoder_layer_attention_beside_mlp_small():
     mlp_graph = manager.graph_module.__dict__[names[1]].callable_dynamic
     targets = [n.target for n in mlp_graph.graph.nodes if n.op == "call_function"]
     assert ops.rms_norm in targets and ops.silu_mul in targets
-    # down projection + residual in one launch; as the value the sub-graph returns it may write into offered rows
-    assert targets.count(ops.linear) == 2
+    # gate and up as one GEMM against stacked weights; down projection + residual in one launch (as the value
+    # the sub-graph returns it may write into offered rows)
+    assert targets.count(ops.linear_multi) == 1 and targets.count(ops.linear) == 0
     assert targets.count(ops.linear_add) + targets.count(ops.linear_add_to_output) == 1
     attn_targets = [n.target for n in manager.graph_module.__dict__[names[0]].callable_dynamic.graph.nodes
                     if n.op == "call_function"]
-    assert attn_targets.count(ops.linear) == 3
+    assert attn_targets.count(ops.linear_multi) == 1 and attn_targets.count(ops.linear) == 0   # q, k, v
     assert attn_targets.count(ops.linear_add) + attn_targets.count(ops.linear_add_to_output) == 1
     assert ops.rms_norm in attn_targets
     assert attn_targets.count(ops.rope) == 2

@@ -29,8 +29,13 @@ def test_bf16_mlp_subgraphs_are_fully_lowered():
     split = traced(torch.bfloat16)
     head, stats0 = lower_to_hip(split.submod_0)
     tail, stats1 = lower_to_hip(split.submod_1)
-    assert stats0 == {"linear": 2, "silu_mul": 0} and stats1 == {"linear": 1, "silu_mul": 1, "to_output": 1}
-    assert targets(head) == [ops.linear, ops.linear]
+    assert stats0 == {"linear": 0, "silu_mul": 0, "linear_multi": 1}
+    assert stats1 == {"linear": 1, "silu_mul": 1, "to_output": 1}
+    # gate and up projection of the same activation: one GEMM against the stacked weights, two column ranges
+    import operator
+    assert targets(head) == [ops.linear_multi, operator.getitem, operator.getitem]
+    multi = next(n for n in head.graph.nodes if n.target is ops.linear_multi)
+    assert len(multi.args[1]) == 2 and all(w.op == "placeholder" for w in multi.args[1])
     # the projection that the sub-graph returns may write into output rows offered by the engine
     assert targets(tail) == [ops.silu_mul, ops.linear_to_output]
     silu_mul = next(n for n in tail.graph.nodes if n.target is ops.silu_mul)
@@ -82,7 +87,11 @@ def test_decoder_layer_rope_and_norms_are_lowered():
     names = [getattr(n.target, "__name__", "") for n in captured["gm"].graph.nodes if n.op == "call_function"]
     assert names.count("apply_rope") == 2          # q and k, each ONE node: dynamo does not trace into it
     lowered, stats = lower_to_hip(captured["gm"])
-    assert stats["rope"] == 2 and stats["rms_norm"] == 2 and stats["linear"] == 7
+    assert stats["rope"] == 2 and stats["rms_norm"] == 2
+    # 7 projections: q / k / v and gate / up each become one GEMM against stacked weights
+    assert stats["linear"] == 2 and stats["linear_multi"] == 2
+    multis = [n for n in lowered.graph.nodes if n.target is ops.linear_multi]
+    assert sorted(len(n.args[1]) for n in multis) == [2, 3]
     assert targets(lowered).count(ops.rope) == 2
 
 
