@@ -16,6 +16,8 @@ it deep-copies the sub-``GraphModule`` and replaces
 
 * two or more bf16 ``linear`` nodes of the same activation (q / k / v projections) -> ONE
   ``dynaflow_hip.linear_multi`` against the stacked weights, results as column ranges of one buffer
+* two ``rope`` nodes with the same tables (q and k) -> ``dynaflow_hip.rope_pair`` (one launch when the inputs
+  are neighbouring column ranges of one buffer)
 * the ``linear`` / ``linear_add`` whose result is what the sub-graph returns -> ``*_to_output``
   (writes into rows offered by the engine, so the nano-batch outputs need no concatenation)
 
@@ -301,6 +303,26 @@ def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False) -> tuple[
             graph.erase_node(member)
         stats["linear_multi"] = stats.get("linear_multi", 0) + 1
         stats["linear"] -= len(members)
+
+    # Two rotations with the same tables (q and k of one attention block) -> one operator, which rotates both
+    # in one launch when it finds k's heads right behind q's (the column ranges of a stacked q / k / v product).
+    order = {n: i for i, n in enumerate(graph.nodes)}
+    ropes = [n for n in graph.nodes if n.op == "call_function" and n.target is ops.rope]
+    while len(ropes) >= 2:
+        first, second = ropes[0], ropes[1]
+        ropes = ropes[2:]
+        if first.args[1] is not second.args[1] or first.args[2] is not second.args[2]:
+            continue
+        if any(order[user] < order[second] for user in first.users):
+            continue                                   # the first result is needed before the second input exists
+        with graph.inserting_before(second):
+            pair = graph.call_function(ops.rope_pair, (first.args[0], second.args[0], first.args[1], first.args[2]))
+            parts = [graph.call_function(operator.getitem, (pair, i)) for i in range(2)]
+        for node, part in zip((first, second), parts):
+            part.meta = dict(node.meta)
+            node.replace_all_uses_with(part)
+            graph.erase_node(node)
+        stats["rope_pair"] = stats.get("rope_pair", 0) + 1
 
     # The projection whose result the sub-graph returns (and nothing else reads) may write straight into the
     # rows that the engine offers for the model output; without an offer it behaves like the plain operator.

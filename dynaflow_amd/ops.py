@@ -38,6 +38,7 @@ _lib.define("rms_norm(Tensor x, Tensor weight, float eps) -> Tensor")
 _lib.define("add_rms_norm(Tensor x, Tensor residual, Tensor weight, float eps) -> (Tensor, Tensor)")
 _lib.define("transpose_weight(Tensor w) -> Tensor")
 _lib.define("rope(Tensor t, Tensor cos, Tensor sin) -> Tensor")
+_lib.define("rope_pair(Tensor q, Tensor k, Tensor cos, Tensor sin) -> (Tensor, Tensor)")
 _lib.define("causal_attention(Tensor q, Tensor k, Tensor v) -> Tensor")
 _lib.define("linear_add(Tensor x, Tensor weight, Tensor residual) -> Tensor")
 _lib.define("linear_to_output(Tensor x, Tensor weight) -> Tensor")
@@ -442,7 +443,34 @@ def _rope_impl(t: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
     return out
 
 
+def _rope_pair_impl(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor):
+    """``(rope(q), rope(k))``; when k's heads sit right behind q's in one buffer (column ranges of a stacked
+    q / k / v product) both are rotated by ONE launch over all the heads."""
+    _require_device(q, k, cos, sin)
+    if q.dim() == 4 and k.dim() == 4 and q.dtype == torch.bfloat16 and k.dtype == torch.bfloat16:
+        qs, ld_q = _token_rows(q, "q")
+        ks, ld_k = _token_rows(k, "k")
+        B, S, hq, d = q.shape
+        hk = k.shape[2]
+        adjacent = (qs is q and ks is k and k.shape[:2] == q.shape[:2] and k.shape[3] == d and ld_q == ld_k
+                    and k.data_ptr() == q.data_ptr() + hq * d * q.element_size())
+        if adjacent and q.numel() > 0 and cos.shape == (S, d // 2) and sin.shape == (S, d // 2):
+            lib = _cabi.load()
+            out = torch.empty((B, S, hq + hk, d), dtype=q.dtype, device=q.device)
+            rc = lib.dfhip_rope_bf16(
+                q.data_ptr(), ld_q, out.data_ptr(), (hq + hk) * d, cos.contiguous().data_ptr(),
+                sin.contiguous().data_ptr(), B * S, hq + hk, d, S, _stream(),
+            )
+            _cabi.check("dfhip_rope_bf16", rc)
+            return out[:, :, :hq], out[:, :, hq:]
+    return _rope_impl(q, cos, sin), _rope_impl(k, cos, sin)
+
+
 _lib.impl("rope", _rope_impl, "CUDA")
+_lib.impl("rope_pair", _rope_pair_impl, "CUDA")
+torch.library.register_fake(
+    "dynaflow_hip::rope_pair", lambda q, k, cos, sin: (torch.empty_like(q), torch.empty_like(k)), lib=_lib
+)
 torch.library.register_fake("dynaflow_hip::rope", lambda t, cos, sin: torch.empty_like(t), lib=_lib)
 
 
@@ -706,6 +734,7 @@ rms_norm = torch.ops.dynaflow_hip.rms_norm
 add_rms_norm = torch.ops.dynaflow_hip.add_rms_norm
 transpose_weight = torch.ops.dynaflow_hip.transpose_weight
 rope = torch.ops.dynaflow_hip.rope
+rope_pair = torch.ops.dynaflow_hip.rope_pair
 decode_attention = torch.ops.dynaflow_hip.decode_attention
 causal_attention = torch.ops.dynaflow_hip.causal_attention
 linear_add = torch.ops.dynaflow_hip.linear_add

@@ -340,6 +340,35 @@ def test_rope_against_complex_rotation(ops, B, S, heads, d):
     assert torch.equal(got[:, 0].cpu(), t[:, 0])  # position 0 is the identity
 
 
+def test_rope_pair_and_stacked_projections_have_the_bits_of_the_separate_operators(ops):
+    """q / k / v as one product against stacked weights, then q and k rotated by one launch straight from the
+    column ranges of that product: every result equals the separate operators' bit for bit (k's heads sit
+    right behind q's, so the one-launch path is taken; with separate tensors the operator falls back)."""
+    from dynaflow_amd.decoder import rope_tables
+
+    B, S, hq, hk, d, H = 2, 64, 8, 2, 128, 1024
+    x = randn((B, S, H), 61).bfloat16().cuda()
+    wq, wk, wv = (randn((n, H), 62 + i, 0.03).bfloat16().cuda() for i, n in enumerate((hq * d, hk * d, hk * d)))
+    cos, sin = (t.cuda() for t in rope_tables(S, d, 500000.0))
+    q, k, v = ops.linear_multi(x, [wq, wk, wv])
+    assert q.data_ptr() + hq * d * 2 == k.data_ptr()                 # column ranges of one buffer
+    # the stacked product picks its own kernel plan: equal to the separate products up to the order of the
+    # fp32 additions (a split along K or not), i.e. within a bf16 rounding of the separate results
+    for got, w in ((q, wq), (k, wk), (v, wv)):
+        want = ops.linear(x, w)
+        assert got.shape == want.shape
+        assert rel_err(got.float(), want.float()) < 2 ** -7
+    q4, k4 = q.view(B, S, hq, d), k.view(B, S, hk, d)
+    rq, rk = ops.rope_pair(q4, k4, cos, sin)
+    assert rq.data_ptr() + hq * d * 2 == rk.data_ptr()               # one launch, one buffer
+    assert torch.equal(rq, ops.rope(q4.contiguous(), cos, sin)) and torch.equal(rk, ops.rope(k4.contiguous(), cos, sin))
+    sq, sk = ops.rope_pair(q4.contiguous(), k4.contiguous(), cos, sin)   # separate tensors: two launches
+    assert torch.equal(sq, rq) and torch.equal(sk, rk)
+    # attention reads the token-strided views in place
+    att = ops.causal_attention(rq, rk, v.view(B, S, hk, d))
+    assert torch.equal(att, ops.causal_attention(rq.contiguous(), rk.contiguous(), v.view(B, S, hk, d).contiguous()))
+
+
 @pytest.mark.parametrize("M,N,K", [(7, 24, 64), (128, 128, 128), (50, 264, 192), (128, 1032, 320), (1, 8, 64)])
 def test_weight_streaming_gemm_small_shapes(ops, M, N, K):
     a = randn((M, K), 1).bfloat16()

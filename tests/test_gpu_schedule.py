@@ -441,7 +441,7 @@ def test_decoder_layer_attention_beside_mlp_small():
     assert attn_targets.count(ops.linear_multi) == 1 and attn_targets.count(ops.linear) == 0   # q, k, v
     assert attn_targets.count(ops.linear_add) + attn_targets.count(ops.linear_add_to_output) == 1
     assert ops.rms_norm in attn_targets
-    assert attn_targets.count(ops.rope) == 2
+    assert attn_targets.count(ops.rope_pair) == 1 and attn_targets.count(ops.rope) == 0     # q and k in one launch
     with torch.no_grad():
         split = manager.prepare(batch, [S] * batch)
         y = compiled(idg)

@@ -92,7 +92,8 @@ def test_decoder_layer_rope_and_norms_are_lowered():
     assert stats["linear"] == 2 and stats["linear_multi"] == 2
     multis = [n for n in lowered.graph.nodes if n.target is ops.linear_multi]
     assert sorted(len(n.args[1]) for n in multis) == [2, 3]
-    assert targets(lowered).count(ops.rope) == 2
+    # ... and the two rotations share their tables: one operator for q and k
+    assert stats["rope_pair"] == 1 and targets(lowered).count(ops.rope_pair) == 1 and ops.rope not in targets(lowered)
 
 
 def test_decoder_layer_attention_is_lowered_for_head_dim_128():
