@@ -134,7 +134,8 @@ class SubgraphCompiler(fx.Interpreter):
             self.config.cudagraph_config,
             use_inductor=target in self.inductor_compile_targets,
             use_cudagraph=target in self.cudagraph_targets,
-            lowering_options={"fuse_silu_epilogue": bool(self.config.knob("fuse_silu_epilogue", False))},
+            lowering_options={"fuse_silu_epilogue": bool(self.config.knob("fuse_silu_epilogue", False)),
+                              "stack_projections": bool(self.config.knob("stack_projections", True))},
         )
         backend.callable_dynamic = backend.compile(list(args))
         self.module.__dict__[target] = backend

@@ -108,7 +108,8 @@ def _silu_mul_supported(g: Any) -> bool:
     return False
 
 
-def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False) -> tuple[fx.GraphModule, dict[str, int]]:
+def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False,
+                 stack_projections: bool = True) -> tuple[fx.GraphModule, dict[str, int]]:
     """Return a lowered deep copy of ``gm`` and a count of each rewrite."""
     # registering the operators is a side effect of importing them
     from dynaflow_amd import ops
@@ -283,8 +284,11 @@ def lower_to_hip(gm: fx.GraphModule, fuse_silu_epilogue: bool = False) -> tuple[
 
     # Several bf16 projections of one activation (q / k / v; gate / up when they are not fused with the product)
     # become one GEMM against the stacked weights: narrow products (1024 columns) fill the chip badly on their own.
+    # (``stack_projections=False`` keeps them apart: the stacked weights are a second copy of the members.)
     groups: dict[fx.Node, list[fx.Node]] = {}
     for node in graph.nodes:
+        if not stack_projections:
+            break
         if node.op == "call_function" and node.target is ops.linear and isinstance(node.args[0], fx.Node):
             ex, ew = _example(node.args[0]), _example(node.args[1])
             if (isinstance(ex, torch.Tensor) and ex.dtype == torch.bfloat16 and isinstance(ew, torch.Tensor)
