@@ -764,14 +764,17 @@ int launch_ring224(const void* A, int64_t lda, const void* W, const void* W2, in
 }
 
 
-// ------------------------------------------------------------------ weight-streaming kernel, M <= 128
-// Decode-sized activations (one nano-batch of single-token queries): the GEMM is bound by reading W
-// once from HBM.  Tile 128 (all rows of A) x 128 columns, 4 waves of 64 x 64, K in slabs of 64 through
+// ------------------------------------------------------------------ weight-streaming kernel, M <= 512
+// Decode-sized activations (a nano-batch of single-token queries): the GEMM is bound by reading W
+// once from HBM.  Tile 128 rows x 128 columns, 4 waves of 64 x 64, K in slabs of 64 through
 // a ring of four 32 KiB units (A half + W half of a slab) filled by LDS-DMA, three slabs in flight per
 // workgroup.  K is split over `split_k` workgroups per tile so that about 200 workgroups stream
 // different parts of W at the same time; the parts meet through the same ticket scheme as above.
-// Workgroups of one K part are neighbours (they share the A columns of that part in one XCD's L2).
+// Workgroups of one K part are neighbours (they share the A columns of that part in one XCD's L2),
+// and with more than 128 rows the row tiles of one column tile are direct neighbours: W leaves HBM
+// once and the other row tiles find it in that XCD's L2.
 constexpr int SK_BM = 128, SK_BN = 128, SK_UNITS = 4, SK_UNIT = 32768, SK_LDS = SK_UNITS * SK_UNIT;
+constexpr int SK_MAX_M = 512;
 
 // FUSED: C[M, N] = silu(A W^T) * (A W2^T) (gate and up weights, N = the intermediate size, K not split):
 // a tile is 128 rows x 64 columns, its W half holds, per wave column, 32 gate rows and the 32 matching up
@@ -780,17 +783,20 @@ template <bool FUSED>
 __global__ void __launch_bounds__(RTHREADS)
 gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
                         const uint16_t* __restrict__ W2, uint16_t* __restrict__ C,
-                        int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int tiles_n, int split_k,
-                        float* __restrict__ partials, int* __restrict__ arrivals) {
+                        int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n,
+                        int split_k, float* __restrict__ partials, int* __restrict__ arrivals) {
   constexpr int TILE_N = FUSED ? SK_BN / 2 : SK_BN;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave & 1, wave_n = wave >> 1;
-  const int work = remap_xcd(blockIdx.x, tiles_n * split_k);
-  const int part = work / tiles_n;
-  const int tile = work - part * tiles_n;
-  const int n0 = tile * TILE_N;
+  const int tiles = tiles_m * tiles_n;
+  const int work = remap_xcd(blockIdx.x, tiles * split_k);
+  const int part = work / tiles;
+  const int tile = work - part * tiles;        // column tile major, row tile minor
+  const int tile_n = tile / tiles_m;
+  const int m0 = (tile - tile_n * tiles_m) * SK_BM;
+  const int n0 = tile_n * TILE_N;
   const int slabs_total = K / BK;
   const int slab0 = (int)((int64_t)slabs_total * part / split_k);
   const int KT = (int)((int64_t)slabs_total * (part + 1) / split_k) - slab0;
@@ -802,7 +808,7 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
   for (int t = 0; t < 4; ++t) {
     const int row = (wave * 4 + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-    int ar = row < M ? row : M - 1;
+    const int ar = m0 + row < M ? m0 + row : M - 1;
     a_src[t] = reinterpret_cast<const uint8_t*>(A + (int64_t)ar * lda + chunk * 8);
     if (FUSED) {
       const int block = row >> 5;                       // 32-row block: wave column block/2, (0: gate, 1: up)
@@ -941,7 +947,7 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
         *reinterpret_cast<u32x2*>(fpark + (i * 32 + frow) * FROW + (g * 8 + fhalf * 4) * 2) = v;
       }
     DFHIP_PIN;
-    const int fm_base = wave_m * 64, fn_base = n0 + wave_n * 32;
+    const int fm_base = m0 + wave_m * 64, fn_base = n0 + wave_n * 32;
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
       const int id = p * 64 + lane;
@@ -968,7 +974,7 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
         *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * PROW + (j * 32 + g * 8 + fhalf * 4) * 2) = v;
       }
   DFHIP_PIN;
-  const int m_base = wave_m * 64, n_base = n0 + wave_n * 64;
+  const int m_base = m0 + wave_m * 64, n_base = n0 + wave_n * 64;
 #pragma unroll 4
   for (int p = 0; p < 8; ++p) {
     const int id = p * 64 + lane;
@@ -986,12 +992,13 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
   }
 }
 
-size_t skinny_counter_bytes(int N) { return counter_area((size_t)(N + SK_BN - 1) / SK_BN); }
+size_t skinny_tiles(int M, int N) { return (size_t)((M + SK_BM - 1) / SK_BM) * ((N + SK_BN - 1) / SK_BN); }
+size_t skinny_counter_bytes(int M, int N) { return counter_area(skinny_tiles(M, N)); }
 
 template <bool FUSED>
 int launch_skinny(const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw, void* C, int64_t ldc, int M,
                   int N, int K, int split_k, void* workspace, hipStream_t stream) {
-  if (M > SK_BM || (FUSED && split_k != 1)) return DFHIP_ERR_BAD_SHAPE;
+  if (M > SK_MAX_M || (FUSED && split_k != 1)) return DFHIP_ERR_BAD_SHAPE;
   auto kernel = gemm_bf16_skinny_kernel<FUSED>;
   static bool lds_opted_in = false;   // one flag per instantiation
   if (!lds_opted_in) {
@@ -1001,14 +1008,15 @@ int launch_skinny(const void* A, int64_t lda, const void* W, const void* W2, int
     lds_opted_in = true;
   }
   constexpr int TILE_N = FUSED ? SK_BN / 2 : SK_BN;
+  const int tiles_m = (M + SK_BM - 1) / SK_BM;
   const int tiles_n = (N + TILE_N - 1) / TILE_N;
   int* arrivals = static_cast<int*>(workspace);
   float* partials = nullptr;
-  if (split_k > 1) partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + skinny_counter_bytes(N));
-  hipLaunchKernelGGL(kernel, dim3(tiles_n * split_k), dim3(RTHREADS), SK_LDS, stream,
+  if (split_k > 1) partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + skinny_counter_bytes(M, N));
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * split_k), dim3(RTHREADS), SK_LDS, stream,
                      static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W),
-                     static_cast<const uint16_t*>(W2), static_cast<uint16_t*>(C), M, N, K, lda, ldw, ldc, tiles_n,
-                     split_k, partials, arrivals);
+                     static_cast<const uint16_t*>(W2), static_cast<uint16_t*>(C), M, N, K, lda, ldw, ldc, tiles_m,
+                     tiles_n, split_k, partials, arrivals);
   return dfhip_check_launch();
 }
 
@@ -1079,11 +1087,13 @@ extern "C" int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* spli
   const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
   *variant = 2;
   *split_k = 1;
-  if (M <= SK_BM && M >= 16 && N >= 1024 && K >= 1024) {
-    // decode-sized activations: stream W with about 192 workgroups (measured best over the 8B shapes: more
-    // parts shorten every workgroup's loop below its fixed costs), at least 8 slabs per part
-    const int tiles_n = (N + SK_BN - 1) / SK_BN;
-    int s = (192 + tiles_n / 2) / tiles_n;
+  // decode-sized activations: up to 128 rows always, up to 512 rows while the 128 x 128 tiles fit one round of
+  // 256 workgroups (beyond that the 256 x 256 tiles below move fewer bytes through LDS per flop and win)
+  const int tiles = (int)skinny_tiles(M, N);
+  if ((M <= SK_BM || (M <= SK_MAX_M && tiles <= 256)) && M >= 16 && N >= 1024 && K >= 1024) {
+    // stream W with about 192 workgroups (measured best over the 8B shapes: more parts shorten every
+    // workgroup's loop below its fixed costs), at least 8 slabs per part
+    int s = (192 + tiles / 2) / tiles;
     if (s < 1) s = 1;
     if (s > 16) s = 16;
     while (s > 1 && K / BK < 8 * s) --s;
@@ -1114,10 +1124,9 @@ extern "C" size_t dfhip_gemm_bf16_splitk_workspace_bytes(int M, int N, int split
   if (M < 1 || N < 1 || split_k < 2) return 0;
   const size_t tiles = (size_t)((M + RBM - 1) / RBM) * ((N + RBN - 1) / RBN);
   const size_t ring = counter_area(tiles) + tiles * split_k * (size_t)RBM * RBN * sizeof(float);
-  if (M > SK_BM) return ring;
-  // the weight-streaming kernel (M <= 128) has its own layout; a caller sizes for whichever is used
-  const size_t skinny = skinny_counter_bytes(N) +
-                        (size_t)((N + SK_BN - 1) / SK_BN) * split_k * (size_t)SK_BM * SK_BN * sizeof(float);
+  if (M > SK_MAX_M) return ring;
+  // the weight-streaming kernel (M <= 512) has its own layout; a caller sizes for whichever is used
+  const size_t skinny = skinny_counter_bytes(M, N) + skinny_tiles(M, N) * split_k * (size_t)SK_BM * SK_BN * sizeof(float);
   return ring > skinny ? ring : skinny;
 }
 
@@ -1147,7 +1156,7 @@ extern "C" int dfhip_gemm_bf16_gate_up_silu(const void* A, int64_t lda, const vo
   if (!W_up) return DFHIP_ERR_NULL_POINTER;
   if (int rc = check_args(A, lda, W_gate, ldw, Out, ldo, M, I, K)) return rc;
   if (!dfhip_aligned16(W_up)) return DFHIP_ERR_BAD_ALIGNMENT;
-  if (M <= SK_BM && I >= 1024 && K >= 1024)   // decode-sized activations: stream both weights once
+  if (M <= 2 * SK_BM && I >= 1024 && K >= 1024)   // decode-sized activations: stream both weights once
     return launch_skinny<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, 1, nullptr,
                                static_cast<hipStream_t>(stream));
   if (round_fill(M, I, TBN / 2) > round_fill(M, I, 128) + 0.05)

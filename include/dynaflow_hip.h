@@ -81,8 +81,10 @@ int dfhip_gemm_bf16_nt(const void* A, int64_t lda, const void* W, int64_t ldw, v
  * variant: 0 = 256x256 tile, LDS-DMA ring (the fast path);
  *          5 = 256x224 tile, LDS-DMA ring (chosen when N = 7 * 2^k makes 224-wide
  *              tiles fill the rounds of 256 workgroups better, e.g. N = 14336);
- *          6 = 128x128 tile for M <= 128 (decode-sized activations): W streamed once
- *              through an LDS-DMA ring, K split over workgroups (see _nt_splitk);
+ *          6 = 128x128 tiles for M <= 512 (decode-sized activations): W streamed once
+ *              through an LDS-DMA ring, K split over workgroups (see _nt_splitk); the
+ *              plan picks it up to 128 rows, and up to 512 rows while the tiles fit
+ *              one round of 256 workgroups;
  *          register-staged tiles: 1 = 256x256 / 8 waves, 2 = 128x128 / 4 waves,
  *          3 = 256x128 / 4 waves, 4 = 256x256 / 4 waves. */
 int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
@@ -103,8 +105,8 @@ int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* split_k);
  * at least dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k) bytes) starts
  * with the per-tile arrival counters, which must be ZERO before the first use
  * and are left zero by every launch; launches that may overlap in time need
- * workspaces of their own.  1 <= split_k <= 8 (16 for M <= 128, where the
- * weight-streaming kernel runs), split_k <= K / 64. */
+ * workspaces of their own.  1 <= split_k <= 8 (16 where the plan picks the
+ * weight-streaming kernel, variant 6), split_k <= K / 64. */
 size_t dfhip_gemm_bf16_splitk_workspace_bytes(int M, int N, int split_k);
 int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                               int64_t ldc, int M, int N, int K, int split_k, void* workspace,

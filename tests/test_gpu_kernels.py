@@ -289,13 +289,14 @@ def test_down_projection_shape_uses_split_k_and_matches_unsplit(ops):
 
 
 @pytest.mark.parametrize("M,I,K", [(1, 8, 64), (300, 264, 192), (257, 136, 128), (512, 1408, 512),
-                                   (2048, 14336, 128), (2000, 14328, 192), (128, 2048, 1024), (100, 1032, 1088)])
+                                   (2048, 14336, 128), (2000, 14328, 192), (128, 2048, 1024), (100, 1032, 1088),
+                                   (256, 2048, 1024), (200, 1032, 1088)])
 def test_gate_up_silu_fused_epilogue(ops, M, I, K):
     """One launch for linear, linear, silu, mul.  The epilogue applies the roundings of the separate kernels,
     so the result has the same bits as linear, linear, silu_mul.  The two large shapes take the 256 x (112
     gate + 112 up) tile (I = 7 * 2^k fills the rounds of 256 workgroups), the others the 256 x (128 + 128)
-    tile; (2000, 14328) has ragged tiles in both directions.  The last two (M <= 128) take the weight-streaming
-    kernel with both weights in one 128 x (32 gate + 32 up) x 2 tile."""
+    tile; (2000, 14328) has ragged tiles in both directions.  The last four (M <= 256) take the weight-streaming
+    kernel with both weights in one 128 x (32 gate + 32 up) x 2 tile, the last two in two row tiles."""
     x = randn((M, K), 41).bfloat16()
     wg = randn((I, K), 42, 0.05).bfloat16()
     wu = randn((I, K), 43, 0.05).bfloat16()
@@ -321,7 +322,9 @@ def test_plan_prefers_224_wide_tiles_for_llama_intermediate_size(ops):
     lib = _cabi.load()
     v, s = ctypes.c_int(), ctypes.c_int()
     for shape, want in (((2048, 14336, 4096), (5, 1)), ((8192, 14336, 4096), (0, 1)), ((8192, 4096, 4096), (0, 1)),
-                        ((2048, 4096, 14336), (0, 2)), ((2048, 28672, 8192), (5, 1))):
+                        ((2048, 4096, 14336), (0, 2)), ((2048, 28672, 8192), (5, 1)),
+                        # more than 128 rows: the weight-streaming kernel only while its tiles fit one round
+                        ((512, 14336, 4096), (0, 2)), ((640, 4096, 4096), (0, 4)), ((256, 14336, 4096), (6, 1))):
         assert lib.dfhip_gemm_bf16_plan(*shape, ctypes.byref(v), ctypes.byref(s)) == 0
         assert (v.value, s.value) == want, shape
 
@@ -369,8 +372,10 @@ def test_rope_pair_and_stacked_projections_have_the_bits_of_the_separate_operato
     assert torch.equal(att, ops.causal_attention(rq.contiguous(), rk.contiguous(), v.view(B, S, hk, d).contiguous()))
 
 
-@pytest.mark.parametrize("M,N,K", [(7, 24, 64), (128, 128, 128), (50, 264, 192), (128, 1032, 320), (1, 8, 64)])
+@pytest.mark.parametrize("M,N,K", [(7, 24, 64), (128, 128, 128), (50, 264, 192), (128, 1032, 320), (1, 8, 64),
+                                   (200, 264, 192), (512, 136, 128), (300, 1032, 320)])
 def test_weight_streaming_gemm_small_shapes(ops, M, N, K):
+    """The last three have two to four row tiles of 128 (the last one ragged)."""
     a = randn((M, K), 1).bfloat16()
     w = randn((N, K), 2, 0.05).bfloat16()
     want = from_u16(cref.gemm_nt_bf16(u16(a), u16(w)))
@@ -382,10 +387,13 @@ def test_weight_streaming_gemm_small_shapes(ops, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K,split", [(128, 4096, 4096, 6), (100, 6144, 4096, 4), (128, 14336, 4096, 2),
-                                         (128, 4096, 14336, 6), (16, 1024, 1024, 2)])
+                                         (128, 4096, 14336, 6), (16, 1024, 1024, 2), (256, 4096, 4096, 3),
+                                         (192, 14336, 4096, 1), (300, 4096, 14336, 2), (512, 6144, 4096, 1),
+                                         (384, 4096, 4096, 2)])
 def test_weight_streaming_gemm_decode_shapes(ops, M, N, K, split):
-    """M <= 128: the plan picks the weight-streaming kernel and splits K so that about 200 workgroups stream W;
-    the parts are added in a fixed order, so the result is the same on every run."""
+    """M <= 128, and up to 512 rows while the 128 x 128 tiles fit one round of 256 workgroups: the plan picks
+    the weight-streaming kernel and splits K so that about 200 workgroups stream W; the parts are added in a
+    fixed order, so the result is the same on every run."""
     import ctypes
 
     from dynaflow_amd import _cabi
@@ -408,7 +416,8 @@ def test_weight_streaming_gemm_decode_shapes(ops, M, N, K, split):
 
 
 @pytest.mark.parametrize("M,N,K", [(300, 264, 192), (7, 24, 64), (2048, 14336, 256), (2048, 4096, 256),
-                                   (2048, 4096, 2048), (128, 4096, 4096), (100, 1032, 1088), (2000, 14328, 192)])
+                                   (2048, 4096, 2048), (128, 4096, 4096), (100, 1032, 1088), (2000, 14328, 192),
+                                   (256, 4096, 4096), (300, 1032, 1088)])
 def test_linear_with_residual_epilogue(ops, M, N, K):
     """linear + add in one launch on every kernel the plan can pick (small tile, ring with and without split-K,
     256 x 224 tile, weight-streaming): the epilogue rounds like the two separate kernels, so the bits match."""
