@@ -273,34 +273,31 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   const int KT = (int)((int64_t)slabs_total * (part + 1) / split_k) - slab0;
 
   // DMA sources: instruction t of this wave covers rows (wave*8+t)*8 .. +8 of a half;
-  // lane -> (row, chunk ^ swizzle(row)) so that LDS slot `lane` holds the swizzled chunk
-  const uint8_t* a_src[8];
-  const uint8_t* w_src[8];
+  // lane -> (row, chunk ^ swizzle(row)) so that LDS slot `lane` holds the swizzled chunk.  The address
+  // is a wave-uniform tile base (scalar registers, advanced per slab) plus a 32-bit byte offset per lane.
+  uint32_t a_off[8], w_off[8];
 #pragma unroll
   for (int t = 0; t < 8; ++t) {
     const int row = (wave * 8 + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     int ar = m0 + row; ar = ar < M ? ar : M - 1;   // rows past the edge re-read the last row; never stored
-    a_src[t] = reinterpret_cast<const uint8_t*>(A + (int64_t)ar * lda + chunk * 8);
-    if (FUSED) {
-      // LDS W row r: 64-row block r/64 = 2*wave_n + (0: gate, 1: up); column wave_n*64 + r%64 of the tile
-      const int block = row >> 6;
-      int wr = n0 + (block >> 1) * 64 + (row & 63); wr = wr < N ? wr : N - 1;
-      const uint16_t* base = (block & 1) ? W2 : W;
-      w_src[t] = reinterpret_cast<const uint8_t*>(base + (int64_t)wr * ldw + chunk * 8);
-    } else {
-      int wr = n0 + row; wr = wr < N ? wr : N - 1;
-      w_src[t] = reinterpret_cast<const uint8_t*>(W + (int64_t)wr * ldw + chunk * 8);
-    }
+    a_off[t] = (uint32_t)((int64_t)(ar - m0) * lda * 2 + chunk * 16);
+    // FUSED, LDS W row r: 64-row block r/64 = 2*wave_n + (0: gate, 1: up); column wave_n*64 + r%64 of the
+    // tile.  The rows of this wave's instructions lie in block `wave`: gate for even, up for odd waves.
+    int wr = FUSED ? n0 + (row >> 7) * 64 + (row & 63) : n0 + row;
+    wr = wr < N ? wr : N - 1;
+    w_off[t] = (uint32_t)((int64_t)(wr - n0) * ldw * 2 + chunk * 16);
   }
+  const uint8_t* const a_tile = reinterpret_cast<const uint8_t*>(A + (int64_t)m0 * lda);
+  const uint8_t* const w_tile = reinterpret_cast<const uint8_t*>(((FUSED && (wave & 1)) ? W2 : W) + (int64_t)n0 * ldw);
   const uint32_t wave_lds = wave * 8 * 1024;
   auto dma_a = [&](int t, int slab, int unit) {
     const int s = slab0 + (slab < KT ? slab : KT - 1);
-    dma16(unit * UNIT + wave_lds + t * 1024, a_src[t] + (int64_t)s * (BK * 2));
+    dma16_base(unit * UNIT + wave_lds + t * 1024, a_tile + (int64_t)s * (BK * 2), a_off[t]);
   };
   auto dma_w = [&](int t, int slab, int unit) {
     const int s = slab0 + (slab < KT ? slab : KT - 1);
-    dma16(unit * UNIT + wave_lds + t * 1024, w_src[t] + (int64_t)s * (BK * 2));
+    dma16_base(unit * UNIT + wave_lds + t * 1024, w_tile + (int64_t)s * (BK * 2), w_off[t]);
   };
 
   const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
@@ -348,11 +345,13 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
 #pragma unroll
   for (int idx = 0; idx < 8; ++idx) read_frag(idx, 0, 0, ua, uw);
   for (int kt = 0; kt < KT; ++kt) {
-    // k-step 0: fragments of step 1 behind MFMAs 0..7, DMA of A(kt+2) behind MFMAs 8..15
+    // k-step 0: fragments of step 1 behind MFMAs 0..7, DMA of A(kt+2) behind every other MFMA (four
+    // waves that issue a DMA per MFMA ask more of the vector memory path than it takes per cycle)
 #pragma unroll
     for (int q = 0; q < 16; ++q) {
       mfma(q, 0);
-      if (q < 8) read_frag(q, 1, 1, ua, uw); else dma_a(q - 8, kt + 2, ia);
+      if (q < 8) read_frag(q, 1, 1, ua, uw);
+      if (q % 2 == 1) dma_a(q / 2, kt + 2, ia);
       DFHIP_PIN;
     }
 #pragma unroll
@@ -375,11 +374,13 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
     workgroup_barrier();
     int na = ua + 2; if (na >= NUNITS) na -= NUNITS;
     int nw = uw + 2; if (nw >= NUNITS) nw -= NUNITS;
-    // k-step 3: DMA of W(kt+2) into the unit A(kt) just left, then fragments of slab kt+1, step 0
+    // k-step 3: DMA of W(kt+2) into the unit A(kt) just left behind every other MFMA, fragments of
+    // slab kt+1, step 0 behind MFMAs 8..15
 #pragma unroll
     for (int q = 0; q < 16; ++q) {
       mfma(q, 1);
-      if (q < 8) dma_w(q, kt + 2, iw); else read_frag(q - 8, 0, 0, na, nw);
+      if (q % 2 == 1) dma_w(q / 2, kt + 2, iw);
+      if (q >= 8) read_frag(q - 8, 0, 0, na, nw);
       DFHIP_PIN;
     }
     ua = na; uw = nw;
@@ -565,36 +566,34 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
   const int n0 = (in_panel / rows_in_panel) * OUT_N;
   const int KT = K / BK;
 
-  // DMA sources.  A half: 32 instructions of 8 rows, 8 per wave.  W half: 28 instructions, 7 per wave.
-  const uint8_t* a_src[8];
-  const uint8_t* w_src[7];
+  // DMA sources.  A half: 32 instructions of 8 rows, 8 per wave.  W half: 28 instructions, 7 per wave
+  // (FUSED: 14 of gate rows, then 14 of up rows: waves 0, 1 read W, waves 2, 3 read W2).  The address is a
+  // wave-uniform tile base (scalar registers, advanced per slab) plus a 32-bit byte offset per lane.
+  uint32_t a_off[8], w_off[7];
 #pragma unroll
   for (int t = 0; t < 8; ++t) {
     const int row = (wave * 8 + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     int ar = m0 + row; ar = ar < M ? ar : M - 1;
-    a_src[t] = reinterpret_cast<const uint8_t*>(A + (int64_t)ar * lda + chunk * 8);
+    a_off[t] = (uint32_t)((int64_t)(ar - m0) * lda * 2 + chunk * 16);
   }
 #pragma unroll
   for (int t = 0; t < 7; ++t) {
     const int row = (wave * 7 + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-    if (FUSED) {
-      const bool up = row >= OUT_N;
-      int wr = n0 + (up ? row - OUT_N : row); wr = wr < N ? wr : N - 1;
-      w_src[t] = reinterpret_cast<const uint8_t*>((up ? W2 : W) + (int64_t)wr * ldw + chunk * 8);
-    } else {
-      int wr = n0 + row; wr = wr < N ? wr : N - 1;
-      w_src[t] = reinterpret_cast<const uint8_t*>(W + (int64_t)wr * ldw + chunk * 8);
-    }
+    int wr = n0 + ((FUSED && row >= OUT_N) ? row - OUT_N : row);
+    wr = wr < N ? wr : N - 1;
+    w_off[t] = (uint32_t)((int64_t)(wr - n0) * ldw * 2 + chunk * 16);
   }
+  const uint8_t* const a_tile = reinterpret_cast<const uint8_t*>(A + (int64_t)m0 * lda);
+  const uint8_t* const w_tile = reinterpret_cast<const uint8_t*>(((FUSED && wave >= 2) ? W2 : W) + (int64_t)n0 * ldw);
   auto dma_a = [&](int t, int slab, int unit) {
     const int s = slab < KT ? slab : KT - 1;
-    dma16(unit * UNIT + (wave * 8 + t) * 1024, a_src[t] + (int64_t)s * (BK * 2));
+    dma16_base(unit * UNIT + (wave * 8 + t) * 1024, a_tile + (int64_t)s * (BK * 2), a_off[t]);
   };
   auto dma_w = [&](int t, int slab, int unit) {
     const int s = slab < KT ? slab : KT - 1;
-    dma16(unit * UNIT + (wave * 7 + t) * 1024, w_src[t] + (int64_t)s * (BK * 2));
+    dma16_base(unit * UNIT + (wave * 7 + t) * 1024, w_tile + (int64_t)s * (BK * 2), w_off[t]);
   };
 
   const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
@@ -645,13 +644,15 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
 #pragma unroll
     for (int q = 0; q < 14; ++q) {
       mfma(q, 0);
-      if (q < 9) read_frag(q, 1, 1, ua, uw); else dma_a(q - 9, kt + 2, ia);
+      if (q < 9) read_frag(q, 1, 1, ua, uw);
+      if (q % 3 == 1) dma_a(q / 3, kt + 2, ia);            // pieces 0..4 behind MFMAs 1, 4, 7, 10, 13
       DFHIP_PIN;
     }
 #pragma unroll
     for (int q = 0; q < 14; ++q) {
       mfma(q, 1);
-      if (q < 9) read_frag(q, 2, 0, ua, uw); else if (q < 12) dma_a(q - 4, kt + 2, ia);
+      if (q < 9) read_frag(q, 2, 0, ua, uw);
+      if (q % 5 == 2) dma_a(5 + q / 5, kt + 2, ia);        // pieces 5..7 behind MFMAs 2, 7, 12
       DFHIP_PIN;
     }
 #pragma unroll
@@ -669,17 +670,8 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
 #pragma unroll
     for (int q = 0; q < 14; ++q) {
       mfma(q, 1);
-      if (q < 7) {
-        dma_w(q, kt + 2, iw);
-      } else if (q < 12) {
-        read_frag(q - 7, 0, 0, na, nw);
-      } else if (q == 12) {
-        read_frag(5, 0, 0, na, nw);
-        read_frag(6, 0, 0, na, nw);
-      } else {
-        read_frag(7, 0, 0, na, nw);
-        read_frag(8, 0, 0, na, nw);
-      }
+      if (q % 2 == 0) dma_w(q / 2, kt + 2, iw);            // the 7 pieces behind every other MFMA
+      if (q >= 5) read_frag(q - 5, 0, 0, na, nw);
       DFHIP_PIN;
     }
     ua = na; uw = nw;
@@ -1054,6 +1046,7 @@ int check_args(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, 
   if (!A || !W || !C) return DFHIP_ERR_NULL_POINTER;
   if (M < 1 || N < 1 || K < 1 || K % BK != 0 || N % 8 != 0) return DFHIP_ERR_BAD_SHAPE;
   if (lda < K || ldw < K || ldc < N) return DFHIP_ERR_BAD_STRIDE;
+  if (lda >= (1 << 22) || ldw >= (1 << 22)) return DFHIP_ERR_BAD_STRIDE;   // 256 rows of a tile within 32-bit byte offsets
   if (lda % 8 || ldw % 8 || ldc % 8 || !dfhip_aligned16(A) || !dfhip_aligned16(W) || !dfhip_aligned16(C))
     return DFHIP_ERR_BAD_ALIGNMENT;
   return DFHIP_OK;
