@@ -267,30 +267,28 @@ gemm_fp8_ring_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ 
   const int n0 = (in_panel / rows_in_panel) * TILE_N;
   const int KT = K / FBK;
 
-  const uint8_t* a_src[8];
-  const uint8_t* w_src[8];
+  // DMA addresses: a wave-uniform tile base (scalar registers, advanced per slab) plus a 32-bit byte
+  // offset per lane.  FUSED: rows 0..127 of the W half come from W (waves 0, 1), rows 128..255 from W2.
+  uint32_t a_off[8], w_off[8];
 #pragma unroll
   for (int t = 0; t < 8; ++t) {
     const int row = (wave * 8 + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     int ar = m0 + row; ar = ar < M ? ar : M - 1;
-    a_src[t] = A + (int64_t)ar * lda + chunk * 16;
-    if (FUSED) {
-      int wr = n0 + (row & 127); wr = wr < N ? wr : N - 1;
-      w_src[t] = (row < 128 ? W : W2) + (int64_t)wr * ldw + chunk * 16;
-    } else {
-      int wr = n0 + row; wr = wr < N ? wr : N - 1;
-      w_src[t] = W + (int64_t)wr * ldw + chunk * 16;
-    }
+    a_off[t] = (uint32_t)((int64_t)(ar - m0) * lda + chunk * 16);
+    int wr = n0 + (FUSED ? (row & 127) : row); wr = wr < N ? wr : N - 1;
+    w_off[t] = (uint32_t)((int64_t)(wr - n0) * ldw + chunk * 16);
   }
+  const uint8_t* const a_tile = A + (int64_t)m0 * lda;
+  const uint8_t* const w_tile = ((FUSED && wave >= 2) ? W2 : W) + (int64_t)n0 * ldw;
   const uint32_t wave_lds = wave * 8 * 1024;
   auto dma_a = [&](int t, int slab, int unit) {
     const int s = slab < KT ? slab : KT - 1;
-    dma16(unit * F8_UNIT + wave_lds + t * 1024, a_src[t] + (int64_t)s * FBK);
+    dma16_base(unit * F8_UNIT + wave_lds + t * 1024, a_tile + (int64_t)s * FBK, a_off[t]);
   };
   auto dma_w = [&](int t, int slab, int unit) {
     const int s = slab < KT ? slab : KT - 1;
-    dma16(unit * F8_UNIT + wave_lds + t * 1024, w_src[t] + (int64_t)s * FBK);
+    dma16_base(unit * F8_UNIT + wave_lds + t * 1024, w_tile + (int64_t)s * FBK, w_off[t]);
   };
 
   // a fragment is 32 bytes = chunks c and c^1 with c = 4*ks + 2*(lane/32), swizzled by (row/2)%8
@@ -494,29 +492,30 @@ gemm_fp8_ring224_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
   const int n0 = (in_panel / rows_in_panel) * F8_TBN;
   const int KT = K / FBK;
 
-  const uint8_t* a_src[8];
-  const uint8_t* w_src[7];
+  uint32_t a_off[8], w_off[7];   // byte offsets from the tile's first row; the tile base sits in scalar registers
 #pragma unroll
   for (int t = 0; t < 8; ++t) {
     const int row = (wave * 8 + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     int ar = m0 + row; ar = ar < M ? ar : M - 1;
-    a_src[t] = A + (int64_t)ar * lda + chunk * 16;
+    a_off[t] = (uint32_t)((int64_t)(ar - m0) * lda + chunk * 16);
   }
 #pragma unroll
   for (int t = 0; t < 7; ++t) {
     const int row = (wave * 7 + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     int wr = n0 + row; wr = wr < N ? wr : N - 1;
-    w_src[t] = W + (int64_t)wr * ldw + chunk * 16;
+    w_off[t] = (uint32_t)((int64_t)(wr - n0) * ldw + chunk * 16);
   }
+  const uint8_t* const a_tile = A + (int64_t)m0 * lda;
+  const uint8_t* const w_tile = W + (int64_t)n0 * ldw;
   auto dma_a = [&](int t, int slab, int unit) {
     const int s = slab < KT ? slab : KT - 1;
-    dma16(unit * F8_UNIT + (wave * 8 + t) * 1024, a_src[t] + (int64_t)s * FBK);
+    dma16_base(unit * F8_UNIT + (wave * 8 + t) * 1024, a_tile + (int64_t)s * FBK, a_off[t]);
   };
   auto dma_w = [&](int t, int slab, int unit) {
     const int s = slab < KT ? slab : KT - 1;
-    dma16(unit * F8_UNIT + (wave * 7 + t) * 1024, w_src[t] + (int64_t)s * FBK);
+    dma16_base(unit * F8_UNIT + (wave * 7 + t) * 1024, w_tile + (int64_t)s * FBK, w_off[t]);
   };
 
   const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
@@ -738,6 +737,7 @@ extern "C" int dfhip_gemm_fp8_nt_variant(const void* A, int64_t lda, const void*
   if (!A || !W || !C || !a_scale || !w_scale) return DFHIP_ERR_NULL_POINTER;
   if (M < 1 || N < 1 || K < 1 || K % FBK != 0 || N % 8 != 0) return DFHIP_ERR_BAD_SHAPE;
   if (lda < K || ldw < K || ldc < N) return DFHIP_ERR_BAD_STRIDE;
+  if (lda >= (1 << 23) || ldw >= (1 << 23)) return DFHIP_ERR_BAD_STRIDE;   // 256 rows of a tile within 32-bit byte offsets
   if (lda % 16 || ldw % 16 || ldc % 8 || !dfhip_aligned16(A) || !dfhip_aligned16(W) || !dfhip_aligned16(C) ||
       !dfhip_aligned16(w_scale))
     return DFHIP_ERR_BAD_ALIGNMENT;
@@ -764,6 +764,7 @@ extern "C" int dfhip_gemm_fp8_gate_up_silu_absmax(const void* A, int64_t lda, co
     return DFHIP_ERR_NULL_POINTER;
   if (M < 1 || I < 8 || K < 1 || K % FBK != 0 || I % 8 != 0) return DFHIP_ERR_BAD_SHAPE;
   if (lda < K || ldw < K || ld_act < I) return DFHIP_ERR_BAD_STRIDE;
+  if (lda >= (1 << 23) || ldw >= (1 << 23)) return DFHIP_ERR_BAD_STRIDE;
   if (lda % 16 || ldw % 16 || ld_act % 8 || !dfhip_aligned16(A) || !dfhip_aligned16(W_gate) ||
       !dfhip_aligned16(W_up) || !dfhip_aligned16(act) || !dfhip_aligned16(w_gate_scale) ||
       !dfhip_aligned16(w_up_scale))

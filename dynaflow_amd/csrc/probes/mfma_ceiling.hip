@@ -65,9 +65,10 @@ int main(){
   bf16x8* d; CK(hipMalloc(&d,h.size()*2)); CK(hipMemcpy(d,h.data(),h.size()*2,hipMemcpyHostToDevice));
   float* out; CK(hipMalloc(&out,256*256*4));
   hipEvent_t e0,e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
-  // per iteration and wave: 16 x 32768 flop (KIND 0) = 64 x 8192... both 524288 flop
+  // per iteration and wave, a 128 x 128 tile: 16 x 32768 flop (32x32x16) = 524288; 64 x 16384 (16x16x32) = 1048576;
+  // 16 x 131072 (fp8 32x32x64) = 2097152
   for(int round=0; round<3; ++round) for(int kind=0; kind<3; ++kind){
-    int iters = kind==2 ? 200000 : 400000;   // an fp8 instruction is 4x the flop of a bf16 one at twice the rate   // 256 WG x 4 waves x 4e5 x 524288 flop = 2.1e14 -> ~0.15 s at 1.4 PF; loop launches for ~3 s
+    int iters = kind==0 ? 400000 : 200000;   // an fp8 instruction is 4x the flop of a bf16 one at twice the rate   // 256 WG x 4 waves x 4e5 x 524288 flop = 2.1e14 -> ~0.15 s at 1.4 PF; loop launches for ~3 s
     CK(hipEventRecord(e0));
     for(int rep=0; rep<20; ++rep){
       if(kind==0) hipLaunchKernelGGL((mfma_tile<0>),dim3(256),dim3(256),0,0,d,iters,out);
@@ -75,7 +76,7 @@ int main(){
       else hipLaunchKernelGGL((mfma_tile<2>),dim3(256),dim3(256),0,0,d,iters,out);
     }
     CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1)); float ms; CK(hipEventElapsedTime(&ms,e0,e1));
-    double flops=20.0*256*4*(double)iters*524288.0*(kind==2?4.0:1.0);
+    double flops=20.0*256*4*(double)iters*524288.0*(kind==2?4.0:kind==1?2.0:1.0);
     printf("round %d %s: %.1f ms  %.1f TFLOP/s\n",round,kind==0?"bf16 32x32x16":kind==1?"bf16 16x16x32":"fp8 32x32x64",ms,flops/ms/1e9); fflush(stdout);
   }
   return 0;
