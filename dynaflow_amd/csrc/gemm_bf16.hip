@@ -217,8 +217,10 @@ constexpr int EROW = 272;    // padded row of the epilogue staging area (bytes)
 // 16-byte store / load that is coherent across the XCDs (sc1: written through to, and read
 // from, the memory side instead of the XCD-private L2).  Used for split-K partial blocks so
 // that no L2-wide write-back or invalidate is needed to hand them from one XCD to another.
+// A store of more than 8 bytes reads its data registers for a few cycles after issue and the compiler
+// cannot see that this statement is one: the wait states keep the next write to those registers away.
 DFHIP_DEVICE void store_f32x4_device_coherent(f32x4* p, f32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
 }
 DFHIP_DEVICE f32x4 load_f32x4_device_coherent(const f32x4* p) {
   f32x4 v;
@@ -240,10 +242,17 @@ size_t counter_area(size_t tiles) {
 // FUSED = false: C[M,N] = A W^T.
 // FUSED = true : C[M,N] = silu(A W^T) * (A W2^T) with W = gate weight, W2 = up weight, N = the
 //   intermediate size.  A tile is 256 rows x 128 columns; its "W half" holds 128 gate rows and 128 up
-//   rows arranged so that every wave owns gate AND up accumulators of the same 128x64 block (MFMA
-//   blocks j = 0,1 are gate, j = 2,3 are up): the SiLU*mul happens in registers with the roundings
-//   of the two-kernel path (bf16 projections, bf16 silu, bf16 product) so that the result has the
-//   same bits, and only the product is written.
+//   rows arranged so that every wave owns gate AND up accumulators of the same 128x64 block: the
+//   SiLU*mul happens in registers with the roundings of the two-kernel path (bf16 projections, bf16
+//   silu, bf16 product) so that the result has the same bits, and only the product is written.
+// The products are v_mfma_f32_16x16x32_bf16: a wave's 128 x 128 block is 8 x 8 blocks of 16 x 16, a slab
+// of 64 is two k-steps of 32.  Per flop the instruction reads half as many accumulator registers as the
+// 32x32x16 one; a loop of nothing but this instruction sustains about 15 % more at the package power
+// limit, and this kernel ran 9-10 % faster than its 32x32x16 predecessor with the same ring.
+//   fragment of a 16-row block for k-step ks: lane -> row lane%16, 16-byte chunk 4*ks + lane/16
+//   acc[i][j] (W block j first operand, A block i second): lane holds
+//     C[16 i + lane%16][16 j + 4 (lane/16) + r], r = 0..3
+// FUSED: blocks j = 0..3 are the gate, j = 4..7 the up projection of the same 64 outputs.
 template <bool FUSED>
 __global__ void __launch_bounds__(RTHREADS)
 gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
@@ -256,8 +265,6 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave & 1, wave_n = wave >> 1;
 
-  // tile order: XCD-contiguous ranges, inside a range panels of GROUP_M tile rows, m fastest
-  // with split-K the parts of one tile are neighbours in launch order
   const int work = remap_xcd(blockIdx.x, tiles_m * tiles_n * split_k);
   const int tile = work / split_k;
   const int part = work - tile * split_k;
@@ -267,23 +274,17 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   const int in_panel = tile % per_panel;
   const int m0 = (first_m + in_panel % rows_in_panel) * RBM;
   const int n0 = (in_panel / rows_in_panel) * TILE_N;
-  // this workgroup multiplies slabs [slab0, slab0 + KT) of the K / 64 slabs
   const int slabs_total = K / BK;
   const int slab0 = (int)((int64_t)slabs_total * part / split_k);
   const int KT = (int)((int64_t)slabs_total * (part + 1) / split_k) - slab0;
 
-  // DMA sources: instruction t of this wave covers rows (wave*8+t)*8 .. +8 of a half;
-  // lane -> (row, chunk ^ swizzle(row)) so that LDS slot `lane` holds the swizzled chunk.  The address
-  // is a wave-uniform tile base (scalar registers, advanced per slab) plus a 32-bit byte offset per lane.
   uint32_t a_off[8], w_off[8];
 #pragma unroll
   for (int t = 0; t < 8; ++t) {
     const int row = (wave * 8 + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-    int ar = m0 + row; ar = ar < M ? ar : M - 1;   // rows past the edge re-read the last row; never stored
+    int ar = m0 + row; ar = ar < M ? ar : M - 1;
     a_off[t] = (uint32_t)((int64_t)(ar - m0) * lda * 2 + chunk * 16);
-    // FUSED, LDS W row r: 64-row block r/64 = 2*wave_n + (0: gate, 1: up); column wave_n*64 + r%64 of the
-    // tile.  The rows of this wave's instructions lie in block `wave`: gate for even, up for odd waves.
     int wr = FUSED ? n0 + (row >> 7) * 64 + (row & 63) : n0 + row;
     wr = wr < N ? wr : N - 1;
     w_off[t] = (uint32_t)((int64_t)(wr - n0) * ldw * 2 + chunk * 16);
@@ -300,21 +301,18 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
     dma16_base(unit * UNIT + wave_lds + t * 1024, w_tile + (int64_t)s * (BK * 2), w_off[t]);
   };
 
-  const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
-  int koff[4];
+  const int frow = lane & 15, fquad = lane >> 4, fswz = (frow >> 1) & 7;
+  int koff[2];
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) koff[ks] = ((2 * ks + fhalf) ^ fswz) * 16;
+  for (int ks = 0; ks < 2; ++ks) koff[ks] = ((4 * ks + fquad) ^ fswz) * 16;
   const int a_lane = (wave_m * 128 + frow) * 128, w_lane = (wave_n * 128 + frow) * 128;
 
-  f32x16 acc[4][4];
+  f32x4 acc[8][8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-  // halves in issue order: A(0) W(0) A(1) W(1) A(2) ...; half h lives in unit h % 5
 #pragma unroll
   for (int t = 0; t < 8; ++t) dma_a(t, 0, 0);
 #pragma unroll
@@ -326,61 +324,50 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   wait_vmcnt<16>();   // slab 0 has landed; slab 1 may still be in flight
   workgroup_barrier();
 
-  bf16x8 fa[2][4], fw[2][4];
-  auto read_frag = [&](int idx, int ks, int slot, int unit_a, int unit_w) {  // idx 0..3: A block, 4..7: W block
-    if (idx < 4)
-      fa[slot][idx] = *reinterpret_cast<const bf16x8*>(smem + unit_a * UNIT + a_lane + koff[ks] + idx * 4096);
+  bf16x8 fa[2][8], fw[2][8];
+  // fragments in the order the MFMAs need them: W block 0, A block 0, W blocks 1..7, A blocks 1..7
+  auto read_frag = [&](int pos, int ks, int slot, int unit_a, int unit_w) {
+    const bool is_a = pos == 1 || pos > 8;
+    const int blk = pos == 0 ? 0 : pos == 1 ? 0 : pos <= 8 ? pos - 1 : pos - 8;
+    if (is_a)
+      fa[slot][blk] = *reinterpret_cast<const bf16x8*>(smem + unit_a * UNIT + a_lane + koff[ks] + blk * 2048);
     else
-      fw[slot][idx - 4] = *reinterpret_cast<const bf16x8*>(smem + unit_w * UNIT + w_lane + koff[ks] + (idx - 4) * 4096);
+      fw[slot][blk] = *reinterpret_cast<const bf16x8*>(smem + unit_w * UNIT + w_lane + koff[ks] + blk * 2048);
   };
-  // snake order over the 4 x 4 blocks: one operand changes per instruction (a pure-MFMA loop sustains
-  // about 1 % more at the power limit this way than with both operands changing at the row ends)
-  auto mfma = [&](int q, int slot) {
-    const int i = q >> 2, j = (i & 1) ? 3 - (q & 3) : (q & 3);
-    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
+  auto mfma = [&](int q, int slot) {   // snake over the 8 x 8 blocks: one operand changes per instruction
+    const int i = q >> 3, j = (i & 1) ? 7 - (q & 7) : (q & 7);
+    // written out so that the accumulator stays in its own registers (the compiler otherwise gives result and
+    // addend different registers and moves 64 accumulators around in every iteration)
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fw[slot][j]), "v"(fa[slot][i]));
   };
 
   int ua = 0, uw = 1;   // units of the slab being multiplied
   int ia = 4, iw = 0;   // units that A(kt+2) and W(kt+2) go to
 #pragma unroll
-  for (int idx = 0; idx < 8; ++idx) read_frag(idx, 0, 0, ua, uw);
+  for (int pos = 0; pos < 16; ++pos) read_frag(pos, 0, 0, ua, uw);
   for (int kt = 0; kt < KT; ++kt) {
-    // k-step 0: fragments of step 1 behind MFMAs 0..7, DMA of A(kt+2) behind every other MFMA (four
-    // waves that issue a DMA per MFMA ask more of the vector memory path than it takes per cycle)
+    // k-step 0: the fragments of k-step 1 behind MFMAs 0..15, the DMA of A(kt+2) behind every sixth after that
 #pragma unroll
-    for (int q = 0; q < 16; ++q) {
+    for (int q = 0; q < 64; ++q) {
       mfma(q, 0);
-      if (q < 8) read_frag(q, 1, 1, ua, uw);
-      if (q % 2 == 1) dma_a(q / 2, kt + 2, ia);
-      DFHIP_PIN;
-    }
-#pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      mfma(q, 1);
-      if (q < 8) read_frag(q, 2, 0, ua, uw);
-      DFHIP_PIN;
-    }
-#pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      mfma(q, 0);
-      if (q < 8) read_frag(q, 3, 1, ua, uw);
+      if (q < 16) read_frag(q, 1, 1, ua, uw);
+      else if ((q - 16) % 6 == 0) dma_a((q - 16) / 6, kt + 2, ia);
       DFHIP_PIN;
     }
     // every LDS read of slab kt has been issued; once they have landed its two units are free.
-    // Slab kt+1 must have landed too: A(kt+1) was issued an iteration ago, W(kt+1) in the last
-    // k-step 3; only the 8 instructions of A(kt+2) may still be in flight.
+    // Slab kt+1 must have landed too; only the 8 instructions of A(kt+2) may still be in flight.
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     wait_vmcnt<8>();
     workgroup_barrier();
     int na = ua + 2; if (na >= NUNITS) na -= NUNITS;
     int nw = uw + 2; if (nw >= NUNITS) nw -= NUNITS;
-    // k-step 3: DMA of W(kt+2) into the unit A(kt) just left behind every other MFMA, fragments of
-    // slab kt+1, step 0 behind MFMAs 8..15
+    // k-step 1: the DMA of W(kt+2) into the unit A(kt) just left behind every fourth MFMA, then the
+    // fragments of slab kt+1, k-step 0
 #pragma unroll
-    for (int q = 0; q < 16; ++q) {
+    for (int q = 0; q < 64; ++q) {
       mfma(q, 1);
-      if (q % 2 == 1) dma_w(q / 2, kt + 2, iw);
-      if (q >= 8) read_frag(q - 8, 0, 0, na, nw);
+      if (q < 32) { if (q % 4 == 0) dma_w(q / 4, kt + 2, iw); }
+      else if (q < 48) read_frag(q - 32, 0, 0, na, nw);
       DFHIP_PIN;
     }
     ua = na; uw = nw;
@@ -389,6 +376,7 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   }
   wait_vmcnt<0>();      // the padding halves issued by the last iterations
   workgroup_barrier();  // other waves may still be reading fragments where this wave parks its block
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written their accumulators
 
   if (!FUSED && split_k > 1) {
     // Every part leaves its fp32 block in `partials` and takes a ticket; the part that draws the
@@ -396,15 +384,10 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
     // and writes the tile.  Nobody waits for anybody.
     f32x4* mine = reinterpret_cast<f32x4*>(partials) + ((int64_t)tile * split_k + part) * (64 * RTHREADS) + tid;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-          store_f32x4_device_coherent(mine + ((i * 4 + j) * 4 + g) * RTHREADS, v);
-        }
-    wait_vmcnt<0>();       // the write-through stores have completed before the ticket is drawn
+      for (int j = 0; j < 8; ++j) store_f32x4_device_coherent(mine + (i * 8 + j) * RTHREADS, acc[i][j]);
+    wait_vmcnt<0>();
     __syncthreads();
     int* ticket_cell = reinterpret_cast<int*>(smem);
     if (tid == 0) *ticket_cell = atomicAdd(arrivals + tile, 1);
@@ -412,32 +395,22 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
     const int ticket = *ticket_cell;
     __syncthreads();
     if (ticket != split_k - 1) return;
-    if (tid == 0) atomicExch(arrivals + tile, 0);   // ready for the next launch
-    // add the parts up in part order, 8 chunks (half a row of MFMA blocks) at a time; the own
-    // part is read back like the others so that the accumulators can start from zero
+    if (tid == 0) atomicExch(arrivals + tile, 0);
     const f32x4* all = reinterpret_cast<const f32x4*>(partials) + (int64_t)tile * split_k * (64 * RTHREADS) + tid;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+      for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     for (int p = 0; p < split_k; ++p) {
 #pragma unroll
-      for (int h = 0; h < 8; ++h) {   // chunks 8h .. 8h+7: blocks (i, j) = (h/2, 2*(h%2) + 0..1)
+      for (int i = 0; i < 8; ++i) {
         f32x4 v[8];
 #pragma unroll
-        for (int c = 0; c < 8; ++c) v[c] = load_f32x4_device_coherent(all + ((int64_t)p * 64 + h * 8 + c) * RTHREADS);
+        for (int j = 0; j < 8; ++j) v[j] = load_f32x4_device_coherent(all + ((int64_t)p * 64 + i * 8 + j) * RTHREADS);
 #pragma unroll
-        for (int c = 0; c < 8; ++c) wait_loaded(v[c]);
+        for (int j = 0; j < 8; ++j) wait_loaded(v[j]);
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-          const int i = h >> 1, j = (h & 1) * 2 + (c >> 2), g = c & 3;
-          acc[i][j][4 * g] += v[c][0];
-          acc[i][j][4 * g + 1] += v[c][1];
-          acc[i][j][4 * g + 2] += v[c][2];
-          acc[i][j][4 * g + 3] += v[c][3];
-        }
+        for (int j = 0; j < 8; ++j) acc[i][j] += v[j];
       }
     }
   }
@@ -447,24 +420,22 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
     constexpr int FROW_BYTES = 144;
     uint8_t* park = smem + wave * (128 * FROW_BYTES);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < 4; ++j) {
+        float p[4];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          float p[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            // the roundings of the two-kernel path: bf16 projections, bf16 silu, bf16 product
-            const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][4 * g + e]));
-            const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j + 2][4 * g + e]));
-            p[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
-          }
-          u32x2 v;
-          v[0] = pack2_bf16(p[0], p[1]);
-          v[1] = pack2_bf16(p[2], p[3]);
-          *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * FROW_BYTES + (j * 32 + g * 8 + fhalf * 4) * 2) = v;
+        for (int e = 0; e < 4; ++e) {
+          // the roundings of the two-kernel path: bf16 projections, bf16 silu, bf16 product
+          const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][e]));
+          const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j + 4][e]));
+          p[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
         }
+        u32x2 v;
+        v[0] = pack2_bf16(p[0], p[1]);
+        v[1] = pack2_bf16(p[2], p[3]);
+        *reinterpret_cast<u32x2*>(park + (i * 16 + frow) * FROW_BYTES + (j * 16 + fquad * 4) * 2) = v;
+      }
     DFHIP_PIN;
     const int m_base = m0 + wave_m * 128, n_base = n0 + wave_n * 64;
 #pragma unroll 4
@@ -480,16 +451,14 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
 
   uint8_t* park = smem + wave * (128 * EROW);
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 v;
-        v[0] = pack2_bf16(acc[i][j][4 * g + 0], acc[i][j][4 * g + 1]);
-        v[1] = pack2_bf16(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
-        *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * EROW + (j * 32 + g * 8 + fhalf * 4) * 2) = v;
-      }
+    for (int j = 0; j < 8; ++j) {
+      u32x2 v;
+      v[0] = pack2_bf16(acc[i][j][0], acc[i][j][1]);
+      v[1] = pack2_bf16(acc[i][j][2], acc[i][j][3]);
+      *reinterpret_cast<u32x2*>(park + (i * 16 + frow) * EROW + (j * 16 + fquad * 4) * 2) = v;
+    }
   DFHIP_PIN;
   const int m_base = m0 + wave_m * 128, n_base = n0 + wave_n * 128;
 #pragma unroll 4
@@ -498,7 +467,7 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
     const int row = id >> 4, c = id & 15;
     u32x4 v = *reinterpret_cast<const u32x4*>(park + row * EROW + c * 16);
     const int m = m_base + row, n = n_base + c * 8;
-    if (m < M && n < N) {  // N % 8 == 0
+    if (m < M && n < N) {
       if (W2) {            // not FUSED: W2 is the optional residual [M, N] (leading dimension ldc)
         const u32x4 r = *reinterpret_cast<const u32x4*>(W2 + (int64_t)m * ldc + n);
 #pragma unroll
@@ -522,7 +491,6 @@ int launch_ring(const void* A, int64_t lda, const void* W, const void* W2, int64
   }
   const int tiles_m = (M + RBM - 1) / RBM;
   const int tiles_n = FUSED ? (N + 127) / 128 : (N + RBN - 1) / RBN;
-  // workspace layout: [tiles] arrival counters (padded to 256 bytes), then [tiles][split_k] fp32 blocks
   int* arrivals = static_cast<int*>(workspace);
   float* partials = nullptr;
   if (split_k > 1) {
@@ -538,7 +506,7 @@ int launch_ring(const void* A, int64_t lda, const void* W, const void* W2, int64
 
 // ------------------------------------------------------------------ ring kernel, 256 x 224 tile
 // Same LDS-DMA ring as above with a tile of 256 rows x 224 columns: 4 waves stacked along M, each
-// 64 x 224 = 2 x 7 MFMA blocks (224 accumulator registers).  Column counts that are multiples of
+// 64 x 224 = 4 x 14 MFMA blocks of 16 x 16 (224 accumulator registers).  Column counts that are multiples of
 // 7 * 2^k (Llama's 14336 = 64 * 224) then give a tile count that divides evenly over the 256 CUs
 // (512 tiles instead of 448 of 256 x 256: 2 full rounds instead of 1.75 rounded up to 2).
 // FUSED: the W half holds 112 gate rows then 112 up rows; the wave parks both projections as
@@ -596,19 +564,17 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
     dma16_base(unit * UNIT + (wave * 7 + t) * 1024, w_tile + (int64_t)s * (BK * 2), w_off[t]);
   };
 
-  const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
-  int koff[4];
+  const int frow = lane & 15, fquad = lane >> 4, fswz = (frow >> 1) & 7;
+  int koff[2];
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) koff[ks] = ((2 * ks + fhalf) ^ fswz) * 16;
+  for (int ks = 0; ks < 2; ++ks) koff[ks] = ((4 * ks + fquad) ^ fswz) * 16;
   const int a_lane = (wave * 64 + frow) * 128, w_lane = frow * 128;
 
-  f32x16 acc[2][7];
+  f32x4 acc[4][14];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 7; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    for (int j = 0; j < 14; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
 #pragma unroll
   for (int t = 0; t < 8; ++t) dma_a(t, 0, 0);
@@ -621,44 +587,32 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
   wait_vmcnt<15>();   // slab 0 has landed; slab 1 may still be in flight
   workgroup_barrier();
 
-  bf16x8 fa[2][2], fw[2][7];
-  // fragments in the order the MFMAs need them: A block 0, W blocks 0..6, A block 1
-  auto read_frag = [&](int idx, int ks, int slot, int unit_a, int unit_w) {
-    if (idx == 0 || idx == 8) {
-      const int i = idx >> 3;
-      fa[slot][i] = *reinterpret_cast<const bf16x8*>(smem + unit_a * UNIT + a_lane + koff[ks] + i * 4096);
-    } else {
-      fw[slot][idx - 1] = *reinterpret_cast<const bf16x8*>(smem + unit_w * UNIT + w_lane + koff[ks] + (idx - 1) * 4096);
-    }
+  bf16x8 fa[2][4], fw[2][14];
+  // fragments in the order the MFMAs need them: W block 0, A block 0, W blocks 1..13, A blocks 1..3
+  auto read_frag = [&](int pos, int ks, int slot, int unit_a, int unit_w) {
+    const bool is_a = pos == 1 || pos > 14;
+    const int blk = pos <= 1 ? 0 : pos <= 14 ? pos - 1 : pos - 14;
+    if (is_a)
+      fa[slot][blk] = *reinterpret_cast<const bf16x8*>(smem + unit_a * UNIT + a_lane + koff[ks] + blk * 2048);
+    else
+      fw[slot][blk] = *reinterpret_cast<const bf16x8*>(smem + unit_w * UNIT + w_lane + koff[ks] + blk * 2048);
   };
-  auto mfma = [&](int q, int slot) {   // snake order: second row walks the W blocks backwards
-    const int i = q / 7, j = i ? 6 - q % 7 : q % 7;
-    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
+  auto mfma = [&](int q, int slot) {   // snake order: odd rows walk the W blocks backwards
+    const int i = q / 14, j = (i & 1) ? 13 - q % 14 : q % 14;
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fw[slot][j]), "v"(fa[slot][i]));
   };
 
   int ua = 0, uw = 1;   // units of the slab being multiplied
   int ia = 4, iw = 0;   // units that A(kt+2) and W(kt+2) go to
 #pragma unroll
-  for (int idx = 0; idx < 9; ++idx) read_frag(idx, 0, 0, ua, uw);
+  for (int pos = 0; pos < 18; ++pos) read_frag(pos, 0, 0, ua, uw);
   for (int kt = 0; kt < KT; ++kt) {
+    // k-step 0: the fragments of k-step 1 behind MFMAs 0..17, the DMA of A(kt+2) behind every fourth after that
 #pragma unroll
-    for (int q = 0; q < 14; ++q) {
+    for (int q = 0; q < 56; ++q) {
       mfma(q, 0);
-      if (q < 9) read_frag(q, 1, 1, ua, uw);
-      if (q % 3 == 1) dma_a(q / 3, kt + 2, ia);            // pieces 0..4 behind MFMAs 1, 4, 7, 10, 13
-      DFHIP_PIN;
-    }
-#pragma unroll
-    for (int q = 0; q < 14; ++q) {
-      mfma(q, 1);
-      if (q < 9) read_frag(q, 2, 0, ua, uw);
-      if (q % 5 == 2) dma_a(5 + q / 5, kt + 2, ia);        // pieces 5..7 behind MFMAs 2, 7, 12
-      DFHIP_PIN;
-    }
-#pragma unroll
-    for (int q = 0; q < 14; ++q) {
-      mfma(q, 0);
-      if (q < 9) read_frag(q, 3, 1, ua, uw);
+      if (q < 18) read_frag(q, 1, 1, ua, uw);
+      else if (q >= 20 && q % 4 == 0 && q < 52) dma_a((q - 20) / 4, kt + 2, ia);
       DFHIP_PIN;
     }
     // all LDS reads of slab kt issued; slab kt+1 must have landed, only A(kt+2) may be in flight
@@ -667,11 +621,12 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
     workgroup_barrier();
     int na = ua + 2; if (na >= NUNITS) na -= NUNITS;
     int nw = uw + 2; if (nw >= NUNITS) nw -= NUNITS;
+    // k-step 1: the 7 pieces of W(kt+2) behind every fourth MFMA, then the fragments of slab kt+1, k-step 0
 #pragma unroll
-    for (int q = 0; q < 14; ++q) {
+    for (int q = 0; q < 56; ++q) {
       mfma(q, 1);
-      if (q % 2 == 0) dma_w(q / 2, kt + 2, iw);            // the 7 pieces behind every other MFMA
-      if (q >= 5) read_frag(q - 5, 0, 0, na, nw);
+      if (q < 28) { if (q % 4 == 0) dma_w(q / 4, kt + 2, iw); }
+      else if (q < 46) read_frag(q - 28, 0, 0, na, nw);
       DFHIP_PIN;
     }
     ua = na; uw = nw;
@@ -680,20 +635,19 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
   }
   wait_vmcnt<0>();
   workgroup_barrier();
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written their accumulators
 
   // park 64 rows x 224 columns per wave as bf16, then store whole row pieces
   uint8_t* park = smem + wave * (64 * TROW);
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 7; ++j)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 v;
-        v[0] = pack2_bf16(acc[i][j][4 * g + 0], acc[i][j][4 * g + 1]);
-        v[1] = pack2_bf16(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
-        *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * TROW + (j * 32 + g * 8 + fhalf * 4) * 2) = v;
-      }
+    for (int j = 0; j < 14; ++j) {
+      u32x2 v;
+      v[0] = pack2_bf16(acc[i][j][0], acc[i][j][1]);
+      v[1] = pack2_bf16(acc[i][j][2], acc[i][j][3]);
+      *reinterpret_cast<u32x2*>(park + (i * 16 + frow) * TROW + (j * 16 + fquad * 4) * 2) = v;
+    }
   DFHIP_PIN;
   const int m_base = m0 + wave * 64;
   if (FUSED) {
