@@ -37,8 +37,8 @@ TOKENS, HIDDEN, INTER, SPLITS = 4096, 4096, 14336, 2
 BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E
 # HBM-side bytes per launch, measured with hardware counters; the summaries are under profiles/
-GATE_GEMM_TRAFFIC_BYTES = 429.7e6      # fetch 371.0 MB + write 58.7 MB
-GATE_UP_SILU_TRAFFIC_BYTES = 797.6e6   # fetch 738.9 MB + write 58.7 MB
+GATE_GEMM_TRAFFIC_BYTES = 429.3e6      # fetch 370.6 MB + write 58.7 MB
+GATE_UP_SILU_TRAFFIC_BYTES = 799.3e6   # fetch 740.6 MB + write 58.7 MB
 METRIC = "MLP-layer tokens/s + overlap speedup vs serial, 8B-shape bf16, 1 MI355X"
 
 
