@@ -291,23 +291,21 @@ gemm_fp8_ring_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ 
     dma16_base(unit * F8_UNIT + wave_lds + t * 1024, w_tile + (int64_t)s * FBK, w_off[t]);
   };
 
-  // a fragment is 32 bytes = chunks c and c^1 with c = 4*ks + 2*(lane/32), swizzled by (row/2)%8
-  const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
-  int koff[2][2];
+  // v_mfma_scale_f32_16x16x128_f8f6f4: one instruction covers the 128 bytes of k of a slab.  A fragment of a
+  // 16-row block is 32 bytes per lane = chunks 2*(lane/16) and 2*(lane/16) + 1 of row lane%16, swizzled by
+  // (row/2)%8.  acc[i][j] (W block j first operand, A block i second): lane holds
+  // C[16 i + lane%16][16 j + 4 (lane/16) + r], r = 0..3.
+  const int frow = lane & 15, fquad = lane >> 4, fswz = (frow >> 1) & 7;
+  int koff[2];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) {
-    koff[ks][0] = ((4 * ks + 2 * fhalf) ^ fswz) * 16;
-    koff[ks][1] = ((4 * ks + 2 * fhalf + 1) ^ fswz) * 16;
-  }
+  for (int part = 0; part < 2; ++part) koff[part] = ((2 * fquad + part) ^ fswz) * 16;
   const int a_lane = (wave_m * 128 + frow) * 128, w_lane = (wave_n * 128 + frow) * 128;
 
-  f32x16 acc[4][4];
+  f32x4 acc[8][8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
 #pragma unroll
   for (int t = 0; t < 8; ++t) dma_a(t, 0, 0);
@@ -320,73 +318,98 @@ gemm_fp8_ring_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ 
   wait_vmcnt<16>();
   workgroup_barrier();
 
-  u32x4 fa[2][4][2], fw[2][4][2];   // [slot][block][low/high 16 bytes]
-  auto read_half = [&](int r, int ks, int slot, int unit_a, int unit_w) {  // r 0..7: A, 8..15: W
-    const int blk = (r & 7) >> 1, part = r & 1;
-    if (r < 8)
-      fa[slot][blk][part] = *reinterpret_cast<const u32x4*>(smem + unit_a * F8_UNIT + a_lane + koff[ks][part] + blk * 4096);
-    else
-      fw[slot][blk][part] = *reinterpret_cast<const u32x4*>(smem + unit_w * F8_UNIT + w_lane + koff[ks][part] + blk * 4096);
+  // A whole slab of fragments is 128 registers per operand; both operands double-buffered would not fit.
+  // The slab is multiplied in two column halves instead: W blocks 0..3 (fwa), then W blocks 4..7 (fwb), both
+  // against all eight A blocks.  The A blocks are double-buffered across slabs, each W half is read while the
+  // other one is in use.
+  u32x4 fa[2][8][2], fwa[4][2], fwb[4][2];   // [..][block][low / high 16 bytes]
+  auto read_a = [&](int half_idx, int slot, int unit_a) {   // half_idx 0..15: block half_idx/2, low / high half
+    const int blk = half_idx >> 1, part = half_idx & 1;
+    fa[slot][blk][part] = *reinterpret_cast<const u32x4*>(smem + unit_a * F8_UNIT + a_lane + koff[part] + blk * 2048);
   };
-  auto mfma = [&](int q, int slot) {
-    const int i = q >> 2, j = q & 3;
+  auto read_w = [&](int half_idx, bool second, int unit_w) {   // half_idx 0..7 within the column half
+    const int blk = half_idx >> 1, part = half_idx & 1;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(smem + unit_w * F8_UNIT + w_lane + koff[part] + ((second ? 4 : 0) + blk) * 2048);
+    if (second) fwb[blk][part] = v; else fwa[blk][part] = v;
+  };
+  const int unit_scale = 0x7f7f7f7f;   // e8m0 scales 2^0
+  auto mfma = [&](int q, int slot, bool second) {   // snake over 8 A blocks x 4 W blocks
+    const int i = q >> 2, jj = (i & 1) ? 3 - (q & 3) : (q & 3);
+    const u32x4 (&w)[2] = second ? fwb[jj] : fwa[jj];
     const i32x8 av = {(int)fa[slot][i][0][0], (int)fa[slot][i][0][1], (int)fa[slot][i][0][2], (int)fa[slot][i][0][3],
                       (int)fa[slot][i][1][0], (int)fa[slot][i][1][1], (int)fa[slot][i][1][2], (int)fa[slot][i][1][3]};
-    const i32x8 wv = {(int)fw[slot][j][0][0], (int)fw[slot][j][0][1], (int)fw[slot][j][0][2], (int)fw[slot][j][0][3],
-                      (int)fw[slot][j][1][0], (int)fw[slot][j][1][1], (int)fw[slot][j][1][2], (int)fw[slot][j][1][3]};
-    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wv, av, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+    const i32x8 wv = {(int)w[0][0], (int)w[0][1], (int)w[0][2], (int)w[0][3], (int)w[1][0], (int)w[1][1], (int)w[1][2], (int)w[1][3]};
+    // written out so that the accumulator keeps its registers
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0]"
+                 : "+a"(acc[i][second ? 4 + jj : jj]) : "v"(wv), "v"(av), "v"(unit_scale));
+  };
+  // reads of the next slab in the order its first MFMAs need them: W block 0, A block 0, W blocks 1..3, A 1..7
+  auto read_next = [&](int pos, int slot, int unit_a, int unit_w) {   // pos 0..23 (fragment halves)
+    if (pos < 2) read_w(pos, false, unit_w);
+    else if (pos < 4) read_a(pos - 2, slot, unit_a);
+    else if (pos < 10) read_w(pos - 2, false, unit_w);
+    else read_a(pos - 8, slot, unit_a);
   };
 
   int ua = 0, uw = 1, ia = 4, iw = 0;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) read_half(r, 0, 0, ua, uw);
-  for (int kt = 0; kt < KT; ++kt) {
-    // k-step 0: one fragment half of step 1 behind every MFMA, DMA of A(kt+2) behind every other one
+  for (int pos = 0; pos < 24; ++pos) read_next(pos, 0, ua, uw);
+  // one slab; `sl` (0 / 1, a constant at each call) is the A fragment buffer this slab multiplies from
+  auto slab = [&](int kt, int sl) {
+    // first column half: the fragments of W blocks 4..7 behind MFMAs 0..7, the DMA of A(kt+2) behind every
+    // other MFMA after that
 #pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      mfma(q, 0);
-      read_half(q, 1, 1, ua, uw);
-      if (q & 1) dma_a(q >> 1, kt + 2, ia);
+    for (int q = 0; q < 32; ++q) {
+      mfma(q, sl, false);
+      if (q < 8) read_w(q, true, uw);
+      else if (q % 2 == 0 && q < 24) dma_a((q - 8) / 2, kt + 2, ia);
       DFHIP_PIN;
     }
+    // every LDS read of slab kt has been issued; slab kt+1 must have landed, only A(kt+2) may be in flight
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     wait_vmcnt<8>();
     workgroup_barrier();
     int na = ua + 2; if (na >= F8_NUNITS) na -= F8_NUNITS;
     int nw = uw + 2; if (nw >= F8_NUNITS) nw -= F8_NUNITS;
-    // k-step 1: DMA of W(kt+2) and the fragments of slab kt+1, step 0
+    // second column half: the DMA of W(kt+2) behind every other MFMA, the 24 fragment halves of slab kt+1
+    // (all of A, W blocks 0..3) behind the others
 #pragma unroll
-    for (int q = 0; q < 16; ++q) {
-      mfma(q, 1);
-      if (!(q & 1)) dma_w(q >> 1, kt + 2, iw);
-      read_half(q, 0, 0, na, nw);
+    for (int q = 0; q < 32; ++q) {
+      mfma(q, sl, true);
+      if (q < 16) { if (q % 2 == 0) dma_w(q / 2, kt + 2, iw); else read_next(q / 2, sl ^ 1, na, nw); }
+      else read_next(8 + (q - 16), sl ^ 1, na, nw);
       DFHIP_PIN;
     }
     ua = na; uw = nw;
     ia += 2; if (ia >= F8_NUNITS) ia -= F8_NUNITS;
     iw += 2; if (iw >= F8_NUNITS) iw -= F8_NUNITS;
+  };
+  int kt = 0;
+  for (; kt + 1 < KT; kt += 2) {
+    slab(kt, 0);
+    slab(kt + 1, 1);
   }
+  if (kt < KT) slab(kt, 0);
   wait_vmcnt<0>();
   workgroup_barrier();
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written their accumulators
 
   // scale, round to bf16, park the wave's 128x128 block in LDS, store whole 256-byte row pieces
   const float sa = a_scale[0];
   uint8_t* park = smem + wave * (128 * F8_EROW);
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int j = 0; j < 8; ++j) {
+    int n = n0 + (FUSED ? 0 : wave_n * 128) + j * 16 + fquad * 4;
+    n = n < N ? n : N - 4;   // columns past the edge are never stored; keep the scale load in bounds
+    const f32x4 ws = *reinterpret_cast<const f32x4*>((FUSED && wave_n ? w2_scale : w_scale) + n);
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      int n = n0 + (FUSED ? 0 : wave_n * 128) + j * 32 + g * 8 + fhalf * 4;
-      n = n < N ? n : N - 4;   // columns past the edge are never stored; keep the scale load in bounds
-      const f32x4 ws = *reinterpret_cast<const f32x4*>((FUSED && wave_n ? w2_scale : w_scale) + n);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        u32x2 v;
-        v[0] = pack2_bf16(acc[i][j][4 * g + 0] * (sa * ws[0]), acc[i][j][4 * g + 1] * (sa * ws[1]));
-        v[1] = pack2_bf16(acc[i][j][4 * g + 2] * (sa * ws[2]), acc[i][j][4 * g + 3] * (sa * ws[3]));
-        *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * F8_EROW + (j * 32 + g * 8 + fhalf * 4) * 2) = v;
-      }
+    for (int i = 0; i < 8; ++i) {
+      u32x2 v;
+      v[0] = pack2_bf16(acc[i][j][0] * (sa * ws[0]), acc[i][j][1] * (sa * ws[1]));
+      v[1] = pack2_bf16(acc[i][j][2] * (sa * ws[2]), acc[i][j][3] * (sa * ws[3]));
+      *reinterpret_cast<u32x2*>(park + (i * 16 + frow) * F8_EROW + (j * 16 + fquad * 4) * 2) = v;
     }
+  }
   DFHIP_PIN;
   if (FUSED) {
     // gate blocks sit in the parks of waves 0, 1 (rows 0..127, 128..255), up blocks in those of waves 2, 3;
@@ -471,7 +494,7 @@ int launch_fp8_ring_fused(const void* A, int64_t lda, const void* Wg, const void
 
 
 // ------------------------------------------------------------------ fp8 ring kernel, 256 x 224 tile
-// The same ring with 4 waves stacked along M, each 64 x 224 = 2 x 7 MFMA blocks: column counts of
+// The same ring with 4 waves stacked along M, each 64 x 224 = 4 x 14 MFMA blocks: column counts of
 // the form 7 * 2^k (28672 = 128 * 224) then fill the rounds of 256 workgroups exactly.
 constexpr int F8_TBN = 224, F8_TROW = F8_TBN * 2 + 16;
 
@@ -518,22 +541,19 @@ gemm_fp8_ring224_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
     dma16_base(unit * F8_UNIT + (wave * 7 + t) * 1024, w_tile + (int64_t)s * FBK, w_off[t]);
   };
 
-  const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
-  int koff[2][2];
+  // fragments and accumulators as in gemm_fp8_ring_kernel (16x16x128 instruction); the slab is multiplied in
+  // two column halves of 7 W blocks against the wave's 4 A blocks
+  const int frow = lane & 15, fquad = lane >> 4, fswz = (frow >> 1) & 7;
+  int koff[2];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) {
-    koff[ks][0] = ((4 * ks + 2 * fhalf) ^ fswz) * 16;
-    koff[ks][1] = ((4 * ks + 2 * fhalf + 1) ^ fswz) * 16;
-  }
+  for (int part = 0; part < 2; ++part) koff[part] = ((2 * fquad + part) ^ fswz) * 16;
   const int a_lane = (wave * 64 + frow) * 128, w_lane = frow * 128;
 
-  f32x16 acc[2][7];
+  f32x4 acc[4][14];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 7; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    for (int j = 0; j < 14; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
 #pragma unroll
   for (int t = 0; t < 8; ++t) dma_a(t, 0, 0);
@@ -546,41 +566,44 @@ gemm_fp8_ring224_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
   wait_vmcnt<15>();
   workgroup_barrier();
 
-  u32x4 fa[2][2][2], fw[2][7][2];   // [slot][block][low/high 16 bytes]
-  // 18 fragment halves in the order the MFMAs need them: A block 0, W blocks 0..6, A block 1
-  auto read_half = [&](int r, int ks, int slot, int unit_a, int unit_w) {
-    const int f = r >> 1, part = r & 1;
-    if (f == 0 || f == 8) {
-      const int i = f >> 3;
-      fa[slot][i][part] = *reinterpret_cast<const u32x4*>(smem + unit_a * F8_UNIT + a_lane + koff[ks][part] + i * 4096);
-    } else {
-      fw[slot][f - 1][part] =
-          *reinterpret_cast<const u32x4*>(smem + unit_w * F8_UNIT + w_lane + koff[ks][part] + (f - 1) * 4096);
-    }
+  u32x4 fa[2][4][2], fwa[7][2], fwb[7][2];   // [..][block][low / high 16 bytes]
+  auto read_a = [&](int half_idx, int slot, int unit_a) {
+    const int blk = half_idx >> 1, part = half_idx & 1;
+    fa[slot][blk][part] = *reinterpret_cast<const u32x4*>(smem + unit_a * F8_UNIT + a_lane + koff[part] + blk * 2048);
   };
-  auto mfma = [&](int q, int slot) {
-    const int i = q / 7, j = q % 7;
+  auto read_w = [&](int half_idx, bool second, int unit_w) {   // half_idx 0..13 within the column half
+    const int blk = half_idx >> 1, part = half_idx & 1;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(smem + unit_w * F8_UNIT + w_lane + koff[part] + ((second ? 7 : 0) + blk) * 2048);
+    if (second) fwb[blk][part] = v; else fwa[blk][part] = v;
+  };
+  const int unit_scale = 0x7f7f7f7f;   // e8m0 scales 2^0
+  auto mfma = [&](int q, int slot, bool second) {   // snake over 4 A blocks x 7 W blocks
+    const int i = q / 7, jj = (i & 1) ? 6 - q % 7 : q % 7;
+    const u32x4 (&w)[2] = second ? fwb[jj] : fwa[jj];
     const i32x8 av = {(int)fa[slot][i][0][0], (int)fa[slot][i][0][1], (int)fa[slot][i][0][2], (int)fa[slot][i][0][3],
                       (int)fa[slot][i][1][0], (int)fa[slot][i][1][1], (int)fa[slot][i][1][2], (int)fa[slot][i][1][3]};
-    const i32x8 wv = {(int)fw[slot][j][0][0], (int)fw[slot][j][0][1], (int)fw[slot][j][0][2], (int)fw[slot][j][0][3],
-                      (int)fw[slot][j][1][0], (int)fw[slot][j][1][1], (int)fw[slot][j][1][2], (int)fw[slot][j][1][3]};
-    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wv, av, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+    const i32x8 wv = {(int)w[0][0], (int)w[0][1], (int)w[0][2], (int)w[0][3], (int)w[1][0], (int)w[1][1], (int)w[1][2], (int)w[1][3]};
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %3 op_sel_hi:[0,0,0]"
+                 : "+a"(acc[i][second ? 7 + jj : jj]) : "v"(wv), "v"(av), "v"(unit_scale));
+  };
+  // reads of the next slab in the order its first MFMAs need them: W block 0, A block 0, W blocks 1..6, A 1..3
+  auto read_next = [&](int pos, int slot, int unit_a, int unit_w) {   // pos 0..21 (fragment halves)
+    if (pos < 2) read_w(pos, false, unit_w);
+    else if (pos < 4) read_a(pos - 2, slot, unit_a);
+    else if (pos < 16) read_w(pos - 2, false, unit_w);
+    else read_a(pos - 14, slot, unit_a);
   };
 
   int ua = 0, uw = 1, ia = 4, iw = 0;
 #pragma unroll
-  for (int r = 0; r < 18; ++r) read_half(r, 0, 0, ua, uw);
-  for (int kt = 0; kt < KT; ++kt) {
-    // k-step 0: 18 fragment halves of step 1, then the 8 DMA instructions of A(kt+2): 26 side operations
-    // behind 14 MFMAs (two behind each of the first twelve)
+  for (int pos = 0; pos < 22; ++pos) read_next(pos, 0, ua, uw);
+  auto slab = [&](int kt, int sl) {
+    // first column half: the 14 fragment halves of W blocks 7..13 and the 8 DMA instructions of A(kt+2)
 #pragma unroll
-    for (int q = 0; q < 14; ++q) {
-      mfma(q, 0);
-      const int first = q < 12 ? 2 * q : 12 + q, last = q < 11 ? 2 * q + 2 : 13 + q;
-#pragma unroll
-      for (int op = first; op < last; ++op) {
-        if (op < 18) read_half(op, 1, 1, ua, uw); else dma_a(op - 18, kt + 2, ia);
-      }
+    for (int q = 0; q < 28; ++q) {
+      mfma(q, sl, false);
+      if (q < 14) read_w(q, true, uw);
+      if (q % 2 == 1 && q < 16) dma_a(q / 2, kt + 2, ia);
       DFHIP_PIN;
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -588,41 +611,43 @@ gemm_fp8_ring224_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
     workgroup_barrier();
     int na = ua + 2; if (na >= F8_NUNITS) na -= F8_NUNITS;
     int nw = uw + 2; if (nw >= F8_NUNITS) nw -= F8_NUNITS;
-    // k-step 1: the 7 DMA instructions of W(kt+2), then the 18 fragment halves of slab kt+1, step 0
+    // second column half: the 7 DMA instructions of W(kt+2), then the 22 fragment halves of slab kt+1
 #pragma unroll
-    for (int q = 0; q < 14; ++q) {
-      mfma(q, 1);
-      const int first = q < 11 ? 2 * q : 11 + q, last = q < 10 ? 2 * q + 2 : 12 + q;
-#pragma unroll
-      for (int op = first; op < last; ++op) {
-        if (op < 7) dma_w(op, kt + 2, iw); else read_half(op - 7, 0, 0, na, nw);
-      }
+    for (int q = 0; q < 28; ++q) {
+      mfma(q, sl, true);
+      if (q % 2 == 0 && q < 14) dma_w(q / 2, kt + 2, iw);
+      if (q >= 6) read_next(q - 6, sl ^ 1, na, nw);
       DFHIP_PIN;
     }
     ua = na; uw = nw;
     ia += 2; if (ia >= F8_NUNITS) ia -= F8_NUNITS;
     iw += 2; if (iw >= F8_NUNITS) iw -= F8_NUNITS;
+  };
+  int kt = 0;
+  for (; kt + 1 < KT; kt += 2) {
+    slab(kt, 0);
+    slab(kt + 1, 1);
   }
+  if (kt < KT) slab(kt, 0);
   wait_vmcnt<0>();
   workgroup_barrier();
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written their accumulators
 
   const float sa = a_scale[0];
   uint8_t* park = smem + wave * (64 * F8_TROW);
 #pragma unroll
-  for (int j = 0; j < 7; ++j)
+  for (int j = 0; j < 14; ++j) {
+    int n = n0 + j * 16 + fquad * 4;
+    n = n < N ? n : N - 4;
+    const f32x4 ws = *reinterpret_cast<const f32x4*>(w_scale + n);
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      int n = n0 + j * 32 + g * 8 + fhalf * 4;
-      n = n < N ? n : N - 4;
-      const f32x4 ws = *reinterpret_cast<const f32x4*>(w_scale + n);
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        u32x2 v;
-        v[0] = pack2_bf16(acc[i][j][4 * g + 0] * (sa * ws[0]), acc[i][j][4 * g + 1] * (sa * ws[1]));
-        v[1] = pack2_bf16(acc[i][j][4 * g + 2] * (sa * ws[2]), acc[i][j][4 * g + 3] * (sa * ws[3]));
-        *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * F8_TROW + (j * 32 + g * 8 + fhalf * 4) * 2) = v;
-      }
+    for (int i = 0; i < 4; ++i) {
+      u32x2 v;
+      v[0] = pack2_bf16(acc[i][j][0] * (sa * ws[0]), acc[i][j][1] * (sa * ws[1]));
+      v[1] = pack2_bf16(acc[i][j][2] * (sa * ws[2]), acc[i][j][3] * (sa * ws[3]));
+      *reinterpret_cast<u32x2*>(park + (i * 16 + frow) * F8_TROW + (j * 16 + fquad * 4) * 2) = v;
     }
+  }
   DFHIP_PIN;
   const int m_base = m0 + wave * 64;
 #pragma unroll 4
