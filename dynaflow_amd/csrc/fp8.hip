@@ -2,15 +2,16 @@
 // and the fp8 GEMM  C = bf16(a_scale * w_scale[n] * A[M,K] * W[N,K]^T).
 //
 // The GEMMs have the byte geometry of the bf16 ones (a K slab row is 128 bytes, here
-// 128 fp8 values) and multiply with v_mfma_scale_f32_32x32x64_f8f6f4 (scale exponents
-// fixed at 2^0), which retires 64 k per instruction - twice the bf16 rate.  A lane
-// feeds 32 consecutive bytes of one row; both operands use the same lane->k mapping,
-// so the contraction is exact whatever order the hardware walks those bytes in.
+// 128 fp8 values) and multiply with the scaled fp8 MFMAs (scale exponents fixed at 2^0):
+// v_mfma_scale_f32_16x16x128_f8f6f4 in the ring kernels, ..._32x32x64_... in the
+// register-staged one - twice the bf16 rate.  A lane feeds 32 consecutive bytes of one
+// row; both operands use the same lane->k mapping, so the contraction is exact whatever
+// order the hardware walks those bytes in.
 //
 // gemm_fp8_ring_kernel  256x256 tile, the LDS-DMA ring / pinned-schedule design of the
 //                       bf16 ring kernel: five 32 KiB LDS units, 1.5 slabs in flight,
 //                       XOR-swizzled 128-byte rows, one LDS read or DMA issue behind every
-//                       MFMA, barrier between the two k-steps of a slab, staged epilogue.
+//                       MFMA, barrier between the two column halves of a slab, staged epilogue.
 // gemm_fp8_nt_kernel    register-staged double buffer for small shapes.
 #include "dfhip_common.h"
 

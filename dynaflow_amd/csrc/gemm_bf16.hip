@@ -1,10 +1,11 @@
 // bf16 GEMM for gfx950:  C[M,N] = A[M,K] * W[N,K]^T, fp32 accumulate, bf16 out.
 //
-// Both operands are K-contiguous, the layout the 32x32x16 bf16 MFMA wants: every
-// lane feeds 8 consecutive k of one row.  The MFMA is issued with W as its first
-// operand and A as its second, i.e. it produces the transposed 32x32 block; in the
-// accumulator layout of v_mfma_f32_32x32x16 a lane then holds ONE row m of C and
-// runs of 4 consecutive columns n.
+// Both operands are K-contiguous, the layout the bf16 MFMAs want: every lane feeds
+// 8 consecutive k of one row.  The MFMA is issued with W as its first operand and A
+// as its second, i.e. it produces the transposed block; in the accumulator layout a
+// lane then holds ONE row m of C and runs of 4 consecutive columns n.  The ring
+// kernels multiply with v_mfma_f32_16x16x32_bf16, the weight-streaming and the
+// register-staged kernels with v_mfma_f32_32x32x16_bf16.
 //
 // Two kernels:
 //
