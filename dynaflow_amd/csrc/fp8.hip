@@ -394,6 +394,12 @@ gemm_fp8_ring_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ 
   wait_vmcnt<0>();
   workgroup_barrier();
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written their accumulators
+  // (the compiler does not know that the statements above write the accumulators late: every later use
+  // of an accumulator is tied behind the wait states)
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
 
   // scale, round to bf16, park the wave's 128x128 block in LDS, store whole 256-byte row pieces
   const float sa = a_scale[0];
@@ -633,6 +639,12 @@ gemm_fp8_ring224_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
   wait_vmcnt<0>();
   workgroup_barrier();
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written their accumulators
+  // (the compiler does not know that the statements above write the accumulators late: every later use
+  // of an accumulator is tied behind the wait states)
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 14; ++j) asm volatile("" : "+a"(acc[i][j]));
 
   const float sa = a_scale[0];
   uint8_t* park = smem + wave * (64 * F8_TROW);

@@ -378,6 +378,12 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   wait_vmcnt<0>();      // the padding halves issued by the last iterations
   workgroup_barrier();  // other waves may still be reading fragments where this wave parks its block
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written their accumulators
+  // (the compiler does not know that the statements above write the accumulators late: every later use
+  // of an accumulator is tied behind the wait states)
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
 
   if (!FUSED && split_k > 1) {
     // Every part leaves its fp32 block in `partials` and takes a ticket; the part that draws the
@@ -637,6 +643,12 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
   wait_vmcnt<0>();
   workgroup_barrier();
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");   // the last MFMAs have written their accumulators
+  // (the compiler does not know that the statements above write the accumulators late: every later use
+  // of an accumulator is tied behind the wait states)
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 14; ++j) asm volatile("" : "+a"(acc[i][j]));
 
   // park 64 rows x 224 columns per wave as bf16, then store whole row pieces
   uint8_t* park = smem + wave * (64 * TROW);
