@@ -516,9 +516,9 @@ int launch_ring(const void* A, int64_t lda, const void* W, const void* W2, int64
 // 64 x 224 = 4 x 14 MFMA blocks of 16 x 16 (224 accumulator registers).  Column counts that are multiples of
 // 7 * 2^k (Llama's 14336 = 64 * 224) then give a tile count that divides evenly over the 256 CUs
 // (512 tiles instead of 448 of 256 x 256: 2 full rounds instead of 1.75 rounded up to 2).
-// FUSED: the W half holds 112 gate rows then 112 up rows; the wave parks both projections as
-// bf16 and the read-back pass computes bf16(bf16(silu(g)) * u) - the roundings of the two-kernel
-// path - and stores the [256, 112] block of the product.
+// FUSED: the W half holds 112 gate rows then 112 up rows, so a lane's accumulators of blocks j and
+// j + 7 are the two projections of the same outputs: bf16(bf16(silu(g)) * u) - the roundings of the
+// two-kernel path - is computed in registers and stored from there, 8 bytes per lane.
 constexpr int TBN = 224;
 constexpr int TROW = TBN * 2 + 16;   // padded row of the staging area (bytes)
 
@@ -650,6 +650,29 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
 #pragma unroll
     for (int j = 0; j < 14; ++j) asm volatile("" : "+a"(acc[i][j]));
 
+  if (FUSED) {
+    // silu(gate) * up in registers (blocks j and j + 7 hold the two projections of the same outputs) and
+    // 8-byte stores straight from the registers: a lane owns 4 consecutive columns of one row
+    const int m_first = m0 + wave * 64 + frow;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 7; ++j) {
+        float p[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][e]));
+          const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j + 7][e]));
+          p[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
+        }
+        u32x2 v;
+        v[0] = pack2_bf16(p[0], p[1]);
+        v[1] = pack2_bf16(p[2], p[3]);
+        const int m = m_first + i * 16, n = n0 + j * 16 + fquad * 4;
+        if (m < M && n < N) *reinterpret_cast<u32x2*>(C + (int64_t)m * ldc + n) = v;
+      }
+    return;
+  }
   // park 64 rows x 224 columns per wave as bf16, then store whole row pieces
   uint8_t* park = smem + wave * (64 * TROW);
 #pragma unroll
@@ -663,27 +686,6 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
     }
   DFHIP_PIN;
   const int m_base = m0 + wave * 64;
-  if (FUSED) {
-#pragma unroll 2
-    for (int p = 0; p < 14; ++p) {
-      const int id = p * 64 + lane;
-      const int row = id / 14, c = id - row * 14;
-      const u32x4 g = *reinterpret_cast<const u32x4*>(park + row * TROW + c * 16);
-      const u32x4 u = *reinterpret_cast<const u32x4*>(park + row * TROW + (14 + c) * 16);
-      u32x4 v;
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        const float g0 = bf16_bits_to_f32(g[w] & 0xffffu), g1 = __uint_as_float(g[w] & 0xffff0000u);
-        const float u0 = bf16_bits_to_f32(u[w] & 0xffffu), u1 = __uint_as_float(u[w] & 0xffff0000u);
-        const float s0 = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(g0)));
-        const float s1 = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(g1)));
-        v[w] = pack2_bf16(s0 * u0, s1 * u1);
-      }
-      const int m = m_base + row, n = n0 + c * 8;
-      if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
-    }
-    return;
-  }
 #pragma unroll 4
   for (int p = 0; p < 28; ++p) {
     const int id = p * 64 + lane;
