@@ -37,7 +37,8 @@ typedef enum dfhip_status {
   DFHIP_OK = 0,
   DFHIP_ERR_NULL_POINTER = -1,
   DFHIP_ERR_BAD_SHAPE = -2,     /* non-positive or unsupported extents */
-  DFHIP_ERR_BAD_STRIDE = -3,    /* leading dimension smaller than the row */
+  DFHIP_ERR_BAD_STRIDE = -3,    /* leading dimension smaller than the row, or of 2^22 (bf16) / 2^23 (fp8)
+                                   elements and more for a GEMM operand */
   DFHIP_ERR_BAD_ALIGNMENT = -4, /* pointer or stride not 16-byte aligned */
   DFHIP_ERR_LAUNCH = -5,        /* hipGetLastError() after the launch */
   DFHIP_ERR_NO_DEVICE = -6,

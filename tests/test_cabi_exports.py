@@ -47,6 +47,9 @@ def test_argument_checks_run_before_any_launch():
     assert lib.dfhip_gemm_bf16_nt(16, 64, 16, 64, 16, 64, 1, 8, 63, None) == -2      # K % 64
     assert lib.dfhip_gemm_bf16_nt(16, 32, 16, 64, 16, 64, 1, 8, 64, None) == -3      # lda < K
     assert lib.dfhip_gemm_bf16_nt(8, 64, 16, 64, 16, 64, 1, 8, 64, None) == -4       # alignment
+    # a tile's 256 rows must stay within 32-bit byte offsets: leading dimensions from 2^22 elements on are refused
+    assert lib.dfhip_gemm_bf16_nt(16, 1 << 22, 16, 64, 16, 64, 1, 8, 64, None) == -3
+    assert lib.dfhip_gemm_bf16_nt(16, 64, 16, 1 << 22, 16, 64, 1, 8, 64, None) == -3
     assert lib.dfhip_gemm_bf16_nt_variant(16, 64, 16, 64, 16, 64, 1, 8, 64, 99, None) == -7
     assert lib.dfhip_silu_mul_bf16(16, 8, 16, 8, 16, 8, 1, 7, 0, None) == -2
     assert lib.dfhip_rmsnorm_bf16(16, None, 16, 16, None, 1, 20000, 1e-5, None) == -2
