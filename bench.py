@@ -287,6 +287,23 @@ def fp8_config(torch, steps, warmup):
                 results[f"{name}_{mode}_ms"] = (time.perf_counter() - t0) * 1e3 / steps
     flops = 6.0 * tokens * hidden * inter
     best = min(results["overlapped_graph_ms"], results["overlapped_fused_gate_up_graph_ms"])
+    # the dominant kernel, alone: gate + up + SiLU*mul + absmax of one nano-batch in one launch
+    from dynaflow_amd import _cabi, ops
+    lib = _cabi.load()
+    mb = tokens // splits
+    with torch.no_grad():
+        xq, xs = ops.quant_fp8(x[:mb])
+    act = torch.empty((mb, inter), dtype=torch.bfloat16, device="cuda")
+    amax = torch.zeros(1, dtype=torch.float32, device="cuda")
+
+    def fused_launch():
+        _cabi.check("dfhip_gemm_fp8_gate_up_silu_absmax", lib.dfhip_gemm_fp8_gate_up_silu_absmax(
+            xq.data_ptr(), hidden, layer.w_gate_q.data_ptr(), layer.w_up_q.data_ptr(), hidden, act.data_ptr(), inter,
+            xs.data_ptr(), layer.w_gate_s.data_ptr(), layer.w_up_s.data_ptr(), amax.data_ptr(), mb, inter, hidden,
+            torch.cuda.current_stream().cuda_stream))
+
+    ms_fused = time_kernel(torch, fused_launch, 30)
+    fused_flops = 4.0 * mb * hidden * inter
     return {
         "metric": "fp8 MLP-layer tokens/s, 70B-shape e4m3, 1 MI355X",
         "value": tokens / (best * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
@@ -297,6 +314,15 @@ def fp8_config(torch, steps, warmup):
                                "the separate gate / up / SiLU*mul launches and the one-launch form is reported"},
         "timings": results,
         "layer": {"tflops": flops / (best * 1e-3) / 1e12, "frac_of_fp8_mfma_peak": flops / (best * 1e-3) / 1e12 / 5000.0},
+        "roofline": {
+            "kernel": "gemm_fp8_ring_kernel<true> (gate and up projection of one nano-batch with the SiLU*mul + absmax "
+                      "epilogue: [2048,8192] x 2 x [28672,8192]^T -> act[2048,28672]), timed alone with HIP events",
+            "bound": "mfma", "achieved": fused_flops / (ms_fused * 1e-3) / 1e12, "peak": 5000.0, "unit": "TFLOP/s",
+            "frac": fused_flops / (ms_fused * 1e-3) / 1e12 / 5000.0, "ms": ms_fused,
+            # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (1410.2 MB fetched + 117.7 MB
+            # written; the summary is under profiles/); algorithmic: 16.8 + 2 x 234.9 MB read, 117.4 MB written
+            "traffic": 1527.9e6, "traffic_unit": "bytes per launch",
+        },
         "overlap_speedup": results["serialized_eager_ms"] / best,
     }
 
@@ -350,6 +376,15 @@ def decoder_config(torch, steps, warmup):
     flops = 2.0 * T * H * 6144 + 2.0 * T * H * H + 2.0 * batch * 32 * S * S * 128 + 6.0 * T * H * I
     best = min(results["overlapped_graph_ms"], results["overlapped_eager_ms"],
                results["overlapped_fused_silu_graph_ms"])
+    # the dominant kernel, alone: gate + up + SiLU*mul of one nano-batch (8192 tokens) in one launch
+    from dynaflow_amd import ops
+    mb = T // 2
+    xb = torch.randn(mb, H, generator=gen, device="cuda", dtype=torch.float32).bfloat16()
+    w_gate = next(p for n, p in layer.named_parameters() if n.endswith("w_gate"))
+    w_up = next(p for n, p in layer.named_parameters() if n.endswith("w_up"))
+    with torch.no_grad():
+        ms_fused = time_kernel(torch, lambda: ops.gate_up_silu(xb, w_gate, w_up), 20)
+    fused_flops = 4.0 * mb * H * I
     return {
         "metric": "decoder-layer prefill tokens/s, 8B-shape bf16, 1 MI355X",
         "value": T / (best * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
@@ -362,6 +397,15 @@ def decoder_config(torch, steps, warmup):
         "timings": results,
         "layer": {"algorithmic_tflop": flops / 1e12, "tflops": flops / (best * 1e-3) / 1e12,
                   "frac_of_bf16_mfma_peak": flops / (best * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS},
+        "roofline": {
+            "kernel": "gemm_bf16_ring_kernel<true> (gate and up projection of one nano-batch with the SiLU*mul "
+                      "epilogue: [8192,4096] x 2 x [14336,4096]^T -> act[8192,14336]), timed alone with HIP events",
+            "bound": "mfma", "achieved": fused_flops / (ms_fused * 1e-3) / 1e12, "peak": BF16_MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s", "frac": fused_flops / (ms_fused * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS, "ms": ms_fused,
+            # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (2821.9 MB fetched + 234.9 MB
+            # written; the summary is under profiles/); algorithmic: 67.1 + 2 x 117.4 MB read, 234.9 MB written
+            "traffic": 3056.8e6, "traffic_unit": "bytes per launch",
+        },
         "overlap_speedup": results["serialized_eager_ms"] / best,
     }
 
