@@ -430,9 +430,12 @@ def decode_config(torch, steps, warmup, layers=32):
     inputs = (ids, slots, lengths)
     half = seqs // 2
     results = {}
+    # the last mode is the comparison without nano-batches: all 256 queries as one batch on one stream (the
+    # weights are read once per step instead of once per nano-batch, nothing overlaps), sub-graphs replayed
     for name, knobs, graphs in (("serialized_eager", {"serialize": True}, False), ("overlapped_eager", {}, False),
                                 ("overlapped_sub_graph_replay", {}, True),
-                                ("stream_per_nano_batch_sub_graph_replay", {"streams": "by_nano_batch"}, True)):
+                                ("stream_per_nano_batch_sub_graph_replay", {"streams": "by_nano_batch"}, True),
+                                ("unsplit_sub_graph_replay", {"min_nano_split_tokens": 1 << 30}, True)):
         extra = {"min_nano_split_tokens": 1, "dump_graph": False, "max_tokens": seqs, "fuse_silu_epilogue": True,
                  **EXTRA_KNOBS}
         extra.update(knobs)
@@ -448,8 +451,9 @@ def decode_config(torch, steps, warmup, layers=32):
             manager.prepare(seqs, [1] * seqs)
             compiled(*inputs)
             if graphs:   # capture every (nano-batch size, nano-batch index) sub-graph in a dry-run
-                manager.prepare(half, [1] * half, is_dryrun=True, use_cudagraph=True)
-                compiled(*(t[:half].contiguous() for t in inputs))
+                size = seqs if name.startswith("unsplit") else half
+                manager.prepare(size, [1] * size, is_dryrun=True, use_cudagraph=True)
+                compiled(*(t[:size].contiguous() for t in inputs))
                 torch.cuda.synchronize()
             for _ in range(warmup):
                 manager.prepare(seqs, [1] * seqs, use_cudagraph=graphs)
@@ -464,7 +468,9 @@ def decode_config(torch, steps, warmup, layers=32):
         del manager, compiled
     weight_bytes = layers * 2.0 * ((heads + 2 * kv_heads) * 128 * H + H * heads * 128 + 3 * H * I)
     kv_bytes = layers * 2.0 * seqs * kv_heads * capacity * 128 * 2
+    unsplit_ms = results.pop("unsplit_sub_graph_replay_ms")
     best = min(results.values())
+    results["unsplit_sub_graph_replay_ms"] = unsplit_ms   # reported beside the nano-batch modes, never as `value`
     return {
         "metric": "decode-step tokens/s, 32 x 8B-shaped layers, bf16, 1 MI355X",
         "value": seqs / (best * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
