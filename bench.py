@@ -592,6 +592,10 @@ def main() -> int:
     ms_fused_graph, yf_graph = time_steps(torch, m_fo, c_fo, x, args.steps, args.warmup, use_graph=True)
     fused_identical = bool(torch.equal(yf_serial, yf_graph))
 
+    # ---- for comparison only: the 4096 tokens as ONE batch (no nano-batches, one stream, two launches)
+    m_un, c_un = build_path(torch, x, weights, min_nano_split_tokens=1 << 30, fuse_silu_epilogue=True)
+    ms_unsplit_gpu = gpu_time_of_steps(torch, m_un, c_un, x, min(args.steps, 20))
+
     # ---- parity of the timed result on sampled rows (fp32 oracle on the same bf16 operands)
     rows = torch.tensor([0, 2047, 2048, 4095])
     want = oracle_mlp.mlp_fp32_from(x_cpu[rows], wg, wu, wd)
@@ -630,6 +634,9 @@ def main() -> int:
             "device": info["arch_name"],
             "compute_units": info["compute_units"],
         },
+        # reported beside the nano-batch schedule, never as `value`: every operator of this layer is MFMA-bound, so
+        # on one GPU two nano-batches have nothing of a different kind to hide behind each other
+        "unsplit_one_batch": {"silu_mul_as_gemm_epilogue_gpu_side_ms": ms_unsplit_gpu},
         "overlap": {
             "serialized_ms": ms_serial,
             "serialized_gpu_side_ms": ms_serial_gpu,
