@@ -725,7 +725,7 @@ int launch_ring224(const void* A, int64_t lda, const void* W, const void* W2, in
 }
 
 
-// ------------------------------------------------------------------ weight-streaming kernel, M <= 512
+// ------------------------------------------------------------------ weight-streaming kernel, M <= 1024
 // Decode-sized activations (a nano-batch of single-token queries): the GEMM is bound by reading W
 // once from HBM.  Tile 128 rows x 128 columns, 4 waves of 64 x 64, K in slabs of 64 through
 // a ring of four 32 KiB units (A half + W half of a slab) filled by LDS-DMA, three slabs in flight per
@@ -735,7 +735,7 @@ int launch_ring224(const void* A, int64_t lda, const void* W, const void* W2, in
 // and with more than 128 rows the row tiles of one column tile are direct neighbours: W leaves HBM
 // once and the other row tiles find it in that XCD's L2.
 constexpr int SK_BM = 128, SK_BN = 128, SK_UNITS = 4, SK_UNIT = 32768, SK_LDS = SK_UNITS * SK_UNIT;
-constexpr int SK_MAX_M = 512;
+constexpr int SK_MAX_M = 1024;
 
 // FUSED: C[M, N] = silu(A W^T) * (A W2^T) (gate and up weights, N = the intermediate size, K not split):
 // a tile is 128 rows x 64 columns, its W half holds, per wave column, 32 gate rows and the 32 matching up
@@ -1049,10 +1049,12 @@ extern "C" int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* spli
   const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
   *variant = 2;
   *split_k = 1;
-  // decode-sized activations: up to 128 rows always, up to 512 rows while the 128 x 128 tiles fit one round of
-  // 256 workgroups (beyond that the 256 x 256 tiles below move fewer bytes through LDS per flop and win)
+  // decode-sized activations: up to 128 rows always, up to 512 rows (1024 with K <= 8192: with a longer K the
+  // 256 x 256 tiles with K split win) while the 128 x 128 tiles fit one round of 256 workgroups; beyond that
+  // the 256 x 256 tiles below move fewer bytes through LDS per flop
   const int tiles = (int)skinny_tiles(M, N);
-  if ((M <= SK_BM || (M <= SK_MAX_M && tiles <= 256)) && M >= 16 && N >= 1024 && K >= 1024) {
+  const bool one_round = tiles <= 256 && (M <= 512 || (M <= SK_MAX_M && K <= 8192));
+  if ((M <= SK_BM || one_round) && M >= 16 && N >= 1024 && K >= 1024) {
     // stream W with about 192 workgroups (measured best over the 8B shapes: more parts shorten every
     // workgroup's loop below its fixed costs), at least 8 slabs per part
     int s = (192 + tiles / 2) / tiles;
@@ -1087,7 +1089,7 @@ extern "C" size_t dfhip_gemm_bf16_splitk_workspace_bytes(int M, int N, int split
   const size_t tiles = (size_t)((M + RBM - 1) / RBM) * ((N + RBN - 1) / RBN);
   const size_t ring = counter_area(tiles) + tiles * split_k * (size_t)RBM * RBN * sizeof(float);
   if (M > SK_MAX_M) return ring;
-  // the weight-streaming kernel (M <= 512) has its own layout; a caller sizes for whichever is used
+  // the weight-streaming kernel (M <= 1024) has its own layout; a caller sizes for whichever is used
   const size_t skinny = skinny_counter_bytes(M, N) + skinny_tiles(M, N) * split_k * (size_t)SK_BM * SK_BN * sizeof(float);
   return ring > skinny ? ring : skinny;
 }

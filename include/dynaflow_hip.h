@@ -82,10 +82,10 @@ int dfhip_gemm_bf16_nt(const void* A, int64_t lda, const void* W, int64_t ldw, v
  * variant: 0 = 256x256 tile, LDS-DMA ring (the fast path);
  *          5 = 256x224 tile, LDS-DMA ring (chosen when N = 7 * 2^k makes 224-wide
  *              tiles fill the rounds of 256 workgroups better, e.g. N = 14336);
- *          6 = 128x128 tiles for M <= 512 (decode-sized activations): W streamed once
+ *          6 = 128x128 tiles for M <= 1024 (decode-sized activations): W streamed once
  *              through an LDS-DMA ring, K split over workgroups (see _nt_splitk); the
- *              plan picks it up to 128 rows, and up to 512 rows while the tiles fit
- *              one round of 256 workgroups;
+ *              plan picks it up to 128 rows, and up to 512 rows (1024 with K <= 8192)
+ *              while the tiles fit one round of 256 workgroups;
  *          register-staged tiles: 1 = 256x256 / 8 waves, 2 = 128x128 / 4 waves,
  *          3 = 256x128 / 4 waves, 4 = 256x256 / 4 waves. */
 int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,

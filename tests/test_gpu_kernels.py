@@ -324,7 +324,8 @@ def test_plan_prefers_224_wide_tiles_for_llama_intermediate_size(ops):
     for shape, want in (((2048, 14336, 4096), (5, 1)), ((8192, 14336, 4096), (0, 1)), ((8192, 4096, 4096), (0, 1)),
                         ((2048, 4096, 14336), (0, 2)), ((2048, 28672, 8192), (5, 1)),
                         # more than 128 rows: the weight-streaming kernel only while its tiles fit one round
-                        ((512, 14336, 4096), (0, 2)), ((640, 4096, 4096), (0, 4)), ((256, 14336, 4096), (6, 1))):
+                        ((512, 14336, 4096), (0, 2)), ((640, 4096, 4096), (6, 1)), ((256, 14336, 4096), (6, 1)),
+                        ((1024, 4096, 4096), (6, 1)), ((1024, 4096, 14336), (0, 4)), ((1024, 6144, 4096), (0, 2))):
         assert lib.dfhip_gemm_bf16_plan(*shape, ctypes.byref(v), ctypes.byref(s)) == 0
         assert (v.value, s.value) == want, shape
 
@@ -389,9 +390,10 @@ def test_weight_streaming_gemm_small_shapes(ops, M, N, K):
 @pytest.mark.parametrize("M,N,K,split", [(128, 4096, 4096, 6), (100, 6144, 4096, 4), (128, 14336, 4096, 2),
                                          (128, 4096, 14336, 6), (16, 1024, 1024, 2), (256, 4096, 4096, 3),
                                          (192, 14336, 4096, 1), (300, 4096, 14336, 2), (512, 6144, 4096, 1),
-                                         (384, 4096, 4096, 2)])
+                                         (384, 4096, 4096, 2), (1000, 4096, 4096, 1)])
 def test_weight_streaming_gemm_decode_shapes(ops, M, N, K, split):
-    """M <= 128, and up to 512 rows while the 128 x 128 tiles fit one round of 256 workgroups: the plan picks
+    """M <= 128, and up to 512 rows (1024 with K <= 8192) while the 128 x 128 tiles fit one round of 256
+    workgroups: the plan picks
     the weight-streaming kernel and splits K so that about 200 workgroups stream W; the parts are added in a
     fixed order, so the result is the same on every run."""
     import ctypes
