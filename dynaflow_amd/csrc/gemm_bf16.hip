@@ -520,14 +520,22 @@ int launch_ring(const void* A, int64_t lda, const void* W, const void* W2, int64
 // j + 7 are the two projections of the same outputs: bf16(bf16(silu(g)) * u) - the roundings of the
 // two-kernel path - is computed in registers and stored from there, 8 bytes per lane.
 constexpr int TBN = 224;
-constexpr int TROW = TBN * 2 + 16;   // padded row of the staging area (bytes)
+// The column count is a template parameter: 224 as described, and 128 (4 x 8 blocks per wave, not FUSED) for
+// shapes whose 256 x 256 tiling has at most half as many tiles as the GPU has CUs - 256 x 128 tiles then fill
+// a round without a split along K and its fp32 partial blocks.
 
-template <bool FUSED>
+template <bool FUSED, int TN>
 __global__ void __launch_bounds__(RTHREADS)
 gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
                          const uint16_t* __restrict__ W2, uint16_t* __restrict__ C,
                          int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n) {
-  constexpr int OUT_N = FUSED ? TBN / 2 : TBN;
+  constexpr int OUT_N = FUSED ? TN / 2 : TN;
+  constexpr int JB = TN / 16;          // 16-column MFMA blocks of a wave: 14 or 8
+  constexpr int WP = TN / 32;          // DMA instructions of a W half per wave: 7 or 4
+  constexpr int NR = 4 + JB;           // fragment reads per k-step
+  constexpr int MQ = 4 * JB;           // MFMAs per k-step
+  constexpr int TROW = TN * 2 + 16;    // padded row of the staging area (bytes)
+  static_assert(!FUSED || TN == TBN, "the fused form exists for the 224-wide tile only");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -544,7 +552,7 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
   // DMA sources.  A half: 32 instructions of 8 rows, 8 per wave.  W half: 28 instructions, 7 per wave
   // (FUSED: 14 of gate rows, then 14 of up rows: waves 0, 1 read W, waves 2, 3 read W2).  The address is a
   // wave-uniform tile base (scalar registers, advanced per slab) plus a 32-bit byte offset per lane.
-  uint32_t a_off[8], w_off[7];
+  uint32_t a_off[8], w_off[WP];
 #pragma unroll
   for (int t = 0; t < 8; ++t) {
     const int row = (wave * 8 + t) * 8 + (lane >> 3);
@@ -553,8 +561,8 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
     a_off[t] = (uint32_t)((int64_t)(ar - m0) * lda * 2 + chunk * 16);
   }
 #pragma unroll
-  for (int t = 0; t < 7; ++t) {
-    const int row = (wave * 7 + t) * 8 + (lane >> 3);
+  for (int t = 0; t < WP; ++t) {
+    const int row = (wave * WP + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     int wr = n0 + ((FUSED && row >= OUT_N) ? row - OUT_N : row);
     wr = wr < N ? wr : N - 1;
@@ -568,7 +576,7 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
   };
   auto dma_w = [&](int t, int slab, int unit) {
     const int s = slab < KT ? slab : KT - 1;
-    dma16_base(unit * UNIT + (wave * 7 + t) * 1024, w_tile + (int64_t)s * (BK * 2), w_off[t]);
+    dma16_base(unit * UNIT + (wave * WP + t) * 1024, w_tile + (int64_t)s * (BK * 2), w_off[t]);
   };
 
   const int frow = lane & 15, fquad = lane >> 4, fswz = (frow >> 1) & 7;
@@ -577,49 +585,50 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
   for (int ks = 0; ks < 2; ++ks) koff[ks] = ((4 * ks + fquad) ^ fswz) * 16;
   const int a_lane = (wave * 64 + frow) * 128, w_lane = frow * 128;
 
-  f32x4 acc[4][14];
+  f32x4 acc[4][JB];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 14; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int j = 0; j < JB; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
 #pragma unroll
   for (int t = 0; t < 8; ++t) dma_a(t, 0, 0);
 #pragma unroll
-  for (int t = 0; t < 7; ++t) dma_w(t, 0, 1);
+  for (int t = 0; t < WP; ++t) dma_w(t, 0, 1);
 #pragma unroll
   for (int t = 0; t < 8; ++t) dma_a(t, 1, 2);
 #pragma unroll
-  for (int t = 0; t < 7; ++t) dma_w(t, 1, 3);
-  wait_vmcnt<15>();   // slab 0 has landed; slab 1 may still be in flight
+  for (int t = 0; t < WP; ++t) dma_w(t, 1, 3);
+  wait_vmcnt<8 + WP>();   // slab 0 has landed; slab 1 may still be in flight
   workgroup_barrier();
 
-  bf16x8 fa[2][4], fw[2][14];
-  // fragments in the order the MFMAs need them: W block 0, A block 0, W blocks 1..13, A blocks 1..3
+  bf16x8 fa[2][4], fw[2][JB];
+  // fragments in the order the MFMAs need them: W block 0, A block 0, W blocks 1.., A blocks 1..3
   auto read_frag = [&](int pos, int ks, int slot, int unit_a, int unit_w) {
-    const bool is_a = pos == 1 || pos > 14;
-    const int blk = pos <= 1 ? 0 : pos <= 14 ? pos - 1 : pos - 14;
+    const bool is_a = pos == 1 || pos > JB;
+    const int blk = pos <= 1 ? 0 : pos <= JB ? pos - 1 : pos - JB;
     if (is_a)
       fa[slot][blk] = *reinterpret_cast<const bf16x8*>(smem + unit_a * UNIT + a_lane + koff[ks] + blk * 2048);
     else
       fw[slot][blk] = *reinterpret_cast<const bf16x8*>(smem + unit_w * UNIT + w_lane + koff[ks] + blk * 2048);
   };
   auto mfma = [&](int q, int slot) {   // snake order: odd rows walk the W blocks backwards
-    const int i = q / 14, j = (i & 1) ? 13 - q % 14 : q % 14;
+    const int i = q / JB, j = (i & 1) ? JB - 1 - q % JB : q % JB;
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fw[slot][j]), "v"(fa[slot][i]));
   };
 
   int ua = 0, uw = 1;   // units of the slab being multiplied
   int ia = 4, iw = 0;   // units that A(kt+2) and W(kt+2) go to
 #pragma unroll
-  for (int pos = 0; pos < 18; ++pos) read_frag(pos, 0, 0, ua, uw);
+  for (int pos = 0; pos < NR; ++pos) read_frag(pos, 0, 0, ua, uw);
   for (int kt = 0; kt < KT; ++kt) {
-    // k-step 0: the fragments of k-step 1 behind MFMAs 0..17, the DMA of A(kt+2) behind every fourth after that
+    // k-step 0: the fragments of k-step 1 behind the first MFMAs, the 8 pieces of A(kt+2) spread over the rest
+    constexpr int A0 = TN == TBN ? NR + 2 : NR, AS = (MQ - A0) / 8;
 #pragma unroll
-    for (int q = 0; q < 56; ++q) {
+    for (int q = 0; q < MQ; ++q) {
       mfma(q, 0);
-      if (q < 18) read_frag(q, 1, 1, ua, uw);
-      else if (q >= 20 && q % 4 == 0 && q < 52) dma_a((q - 20) / 4, kt + 2, ia);
+      if (q < NR) read_frag(q, 1, 1, ua, uw);
+      else if (q >= A0 && (q - A0) % AS == 0 && (q - A0) / AS < 8) dma_a((q - A0) / AS, kt + 2, ia);
       DFHIP_PIN;
     }
     // all LDS reads of slab kt issued; slab kt+1 must have landed, only A(kt+2) may be in flight
@@ -628,12 +637,12 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
     workgroup_barrier();
     int na = ua + 2; if (na >= NUNITS) na -= NUNITS;
     int nw = uw + 2; if (nw >= NUNITS) nw -= NUNITS;
-    // k-step 1: the 7 pieces of W(kt+2) behind every fourth MFMA, then the fragments of slab kt+1, k-step 0
+    // k-step 1: the pieces of W(kt+2) behind every fourth MFMA, then the fragments of slab kt+1, k-step 0
 #pragma unroll
-    for (int q = 0; q < 56; ++q) {
+    for (int q = 0; q < MQ; ++q) {
       mfma(q, 1);
-      if (q < 28) { if (q % 4 == 0) dma_w(q / 4, kt + 2, iw); }
-      else if (q < 46) read_frag(q - 28, 0, 0, na, nw);
+      if (q < 4 * WP) { if (q % 4 == 0) dma_w(q / 4, kt + 2, iw); }
+      else if (q < 4 * WP + NR) read_frag(q - 4 * WP, 0, 0, na, nw);
       DFHIP_PIN;
     }
     ua = na; uw = nw;
@@ -648,7 +657,7 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 14; ++j) asm volatile("" : "+a"(acc[i][j]));
+    for (int j = 0; j < JB; ++j) asm volatile("" : "+a"(acc[i][j]));
 
   if (FUSED) {
     // silu(gate) * up in registers (blocks j and j + 7 hold the two projections of the same outputs) and
@@ -657,12 +666,12 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 7; ++j) {
+      for (int j = 0; j < JB / 2; ++j) {
         float p[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][e]));
-          const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j + 7][e]));
+          const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j + JB / 2][e]));
           p[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
         }
         u32x2 v;
@@ -678,7 +687,7 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 14; ++j) {
+    for (int j = 0; j < JB; ++j) {
       u32x2 v;
       v[0] = pack2_bf16(acc[i][j][0], acc[i][j][1]);
       v[1] = pack2_bf16(acc[i][j][2], acc[i][j][3]);
@@ -686,10 +695,11 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
     }
   DFHIP_PIN;
   const int m_base = m0 + wave * 64;
+  constexpr int CPR = TN / 8;   // 16-byte pieces of a row
 #pragma unroll 4
-  for (int p = 0; p < 28; ++p) {
+  for (int p = 0; p < CPR; ++p) {
     const int id = p * 64 + lane;
-    const int row = id / 28, c = id - row * 28;
+    const int row = id / CPR, c = id - row * CPR;
     u32x4 v = *reinterpret_cast<const u32x4*>(park + row * TROW + c * 16);
     const int m = m_base + row, n = n0 + c * 8;
     if (m < M && n < N) {
@@ -703,18 +713,18 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
   }
 }
 
-template <bool FUSED>
+template <bool FUSED, int TN = TBN>
 int launch_ring224(const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw, void* C, int64_t ldc,
                    int M, int N, int K, hipStream_t stream) {
-  auto kernel = gemm_bf16_ring224_kernel<FUSED>;
-  static bool lds_opted_in = false;
+  auto kernel = gemm_bf16_ring224_kernel<FUSED, TN>;
+  static bool lds_opted_in = false;   // one flag per instantiation
   if (!lds_opted_in) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             RING_LDS) != hipSuccess)
       return DFHIP_ERR_LAUNCH;
     lds_opted_in = true;
   }
-  constexpr int OUT_N = FUSED ? TBN / 2 : TBN;
+  constexpr int OUT_N = FUSED ? TN / 2 : TN;
   const int tiles_m = (M + RBM - 1) / RBM;
   const int tiles_n = (N + OUT_N - 1) / OUT_N;
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(RTHREADS), RING_LDS, stream,
@@ -1035,6 +1045,7 @@ extern "C" int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void
     case 2: return launch<128, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 3: return launch<256, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s);
     case 5: return launch_ring224<false>(A, lda, W, nullptr, ldw, C, ldc, M, N, K, s);
+    case 7: return launch_ring224<false, 128>(A, lda, W, nullptr, ldw, C, ldc, M, N, K, s);
     case 6: return launch_skinny<false>(A, lda, W, nullptr, ldw, C, ldc, M, N, K, 1, nullptr, s);
     default: return DFHIP_ERR_BAD_ARGUMENT;
   }
@@ -1071,6 +1082,13 @@ extern "C" int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* spli
     if (s > 8) s = 8;
     while (s > 1 && K / BK < 16 * s) --s;   // keep at least 16 slabs per part
     if (s > 1) *split_k = s;
+    // few tiles and a short K: 256 x 128 tiles fill the CUs without the fp32 partial blocks of a split
+    // (with K = 14336 the split 256 x 256 tiles are as fast or faster)
+    if (s > 1 && K <= 8192) {
+      *variant = 7;
+      *split_k = 1;
+      return DFHIP_OK;
+    }
     // 256 x 224 tiles when they fill the rounds of 256 workgroups clearly better (N = 7 * 2^k)
     if (s <= 1 && round_fill(M, N, TBN) > round_fill(M, N, RBN) + 0.05) *variant = 5;
   }
@@ -1149,6 +1167,7 @@ extern "C" int dfhip_gemm_bf16_nt_add(const void* A, int64_t lda, const void* W,
   switch (variant) {
     case 0: return launch_ring<false>(A, lda, W, R, ldw, C, ldc, M, N, K, split_k, workspace, s);
     case 5: return launch_ring224<false>(A, lda, W, R, ldw, C, ldc, M, N, K, s);
+    case 7: return launch_ring224<false, 128>(A, lda, W, R, ldw, C, ldc, M, N, K, s);
     case 6: return launch_skinny<false>(A, lda, W, R, ldw, C, ldc, M, N, K, split_k, workspace, s);
     default: return launch<128, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s, R);
   }

@@ -86,6 +86,8 @@ int dfhip_gemm_bf16_nt(const void* A, int64_t lda, const void* W, int64_t ldw, v
  *              through an LDS-DMA ring, K split over workgroups (see _nt_splitk); the
  *              plan picks it up to 128 rows, and up to 512 rows (1024 with K <= 8192)
  *              while the tiles fit one round of 256 workgroups;
+ *          7 = 256x128 tile, LDS-DMA ring (chosen instead of a split along K when the
+ *              256x256 tiling has few tiles and K <= 8192);
  *          register-staged tiles: 1 = 256x256 / 8 waves, 2 = 128x128 / 4 waves,
  *          3 = 256x128 / 4 waves, 4 = 256x256 / 4 waves. */
 int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,

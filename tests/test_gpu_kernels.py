@@ -60,7 +60,7 @@ def test_device_info(ops):
 
 @pytest.mark.parametrize("M,N,K", [(1, 8, 64), (7, 24, 64), (128, 128, 128), (300, 264, 192), (257, 512, 256),
                                    (512, 1032, 320)])
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5, 7])
 def test_gemm_bf16_against_c_oracle(ops, M, N, K, variant):
     a = randn((M, K), 1).bfloat16()
     w = randn((N, K), 2, 0.05).bfloat16()
@@ -324,8 +324,10 @@ def test_plan_prefers_224_wide_tiles_for_llama_intermediate_size(ops):
     for shape, want in (((2048, 14336, 4096), (5, 1)), ((8192, 14336, 4096), (0, 1)), ((8192, 4096, 4096), (0, 1)),
                         ((2048, 4096, 14336), (0, 2)), ((2048, 28672, 8192), (5, 1)),
                         # more than 128 rows: the weight-streaming kernel only while its tiles fit one round
-                        ((512, 14336, 4096), (0, 2)), ((640, 4096, 4096), (6, 1)), ((256, 14336, 4096), (6, 1)),
-                        ((1024, 4096, 4096), (6, 1)), ((1024, 4096, 14336), (0, 4)), ((1024, 6144, 4096), (0, 2))):
+                        ((512, 14336, 4096), (7, 1)), ((640, 4096, 4096), (6, 1)), ((256, 14336, 4096), (6, 1)),
+                        ((1024, 4096, 4096), (6, 1)), ((1024, 4096, 14336), (0, 4)), ((1024, 6144, 4096), (7, 1)),
+                        # few 256 x 256 tiles and a short K: 256 x 128 tiles instead of a split along K
+                        ((2048, 4096, 4096), (7, 1))):
         assert lib.dfhip_gemm_bf16_plan(*shape, ctypes.byref(v), ctypes.byref(s)) == 0
         assert (v.value, s.value) == want, shape
 
