@@ -473,3 +473,55 @@ def test_fp8_gate_up_silu_epilogue_has_the_bits_of_the_separate_operators(ops, M
     assert torch.equal(got_q.view(torch.uint8), want_q.view(torch.uint8))
     again_q, again_s = ops.gate_up_silu_quant_fp8(xq, wgq, wuq, xs, wgs, wus)
     assert torch.equal(again_q.view(torch.uint8), got_q.view(torch.uint8)) and torch.equal(again_s, got_s)
+
+
+def _seeded_shapes(seed, count):
+    import random
+    rng = random.Random(seed)
+    shapes = []
+    for it in range(count):
+        M = rng.choice([1, 17, 128, 129, 255, 256, 257, 511, 513, 700, 1024, 1500, 2048, 3000])
+        N = 8 * rng.randint(1, 600) if it % 3 else rng.choice([224, 448, 896, 1792, 3584, 4096, 6144])
+        K = 64 * rng.randint(1, 40) if it % 2 else rng.choice([64, 128, 192, 4096, 2048])
+        shapes.append((M, N, K))
+    return shapes
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", _seeded_shapes(20261, 24))
+def test_planned_gemm_on_seeded_random_shapes(ops, M, N, K):
+    """Whatever kernel and split the plan picks for a shape (ragged rows and columns, short and long K):
+    `linear` against the fp32 product of the same bf16 operands (tolerance 2^-7 of the largest output: bf16
+    output rounding plus fp32 accumulation order), `linear_add` with the bits of `linear` followed by `add`,
+    and the fused gate/up/SiLU launch with the bits of the three separate launches."""
+    a = randn((M, K), 51).bfloat16().cuda()
+    w = randn((N, K), 52, 0.05).bfloat16().cuda()
+    r = randn((M, N), 53).bfloat16().cuda()
+    want = a.float() @ w.float().t()
+    y = ops.linear(a, w)
+    err = ((y.float() - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+    assert err <= 2.0 ** -7, (M, N, K, err)
+    assert torch.equal(ops.linear_add(a, w, r), r + y)
+    inter = (N // 16) * 8
+    if inter >= 8:
+        wg, wu = w[:inter].contiguous(), w[inter:2 * inter].contiguous()
+        fused = ops.gate_up_silu(a, wg, wu)
+        separate = ops.silu_mul(ops.linear_variant(a, wg, -2), ops.linear_variant(a, wu, -2), True)
+        assert torch.equal(fused, separate)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(1, 8, 128), (100, 3584, 1536), (257, 1808, 384), (1100, 2456, 3072),
+                                   (2048, 224, 2304), (4096, 3000, 640), (256, 8192, 1024), (700, 28672, 256)])
+def test_planned_fp8_gemm_on_assorted_shapes(ops, M, N, K):
+    """e4m3 `linear` with per-tensor activation scale and per-row weight scales against the fp32 product of the
+    dequantised operands (tolerance 2^-6 of the largest output: the bf16 rounding of the output dominates)."""
+    x = randn((M, K), 61).bfloat16().cuda()
+    w = randn((N, K), 62, 0.05).bfloat16().cuda()
+    xq, xs = ops.quant_fp8(x)
+    ws = (w.float().abs().amax(dim=1) / 448.0).clamp_min(1e-12)
+    wq = (w.float() / ws[:, None]).to(torch.float8_e4m3fn)
+    got = ops.linear_fp8(xq, wq, xs, ws)
+    want = (xq.float() * xs) @ (wq.float() * ws[:, None]).t()
+    err = ((got.float() - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+    assert err <= 2.0 ** -6, (M, N, K, err)
