@@ -482,13 +482,8 @@ extern "C" int dfhip_causal_attention_bf16(const void* q, int64_t ld_q, const vo
   if (ld_q % 8 || ld_k % 8 || ld_o % 8 || !dfhip_aligned16(q) || !dfhip_aligned16(k) || !dfhip_aligned16(v_blk) ||
       !dfhip_aligned16(out))
     return DFHIP_ERR_BAD_ALIGNMENT;
-  static bool lds_opted_in = false;
-  if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(causal_attention_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, ATT_LDS) != hipSuccess)
-      return DFHIP_ERR_LAUNCH;
-    lds_opted_in = true;
-  }
+  static std::atomic<uint64_t> lds_opted_in{0};   // per instantiation, one bit per device
+  if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(causal_attention_kernel), ATT_LDS, lds_opted_in)) return rc;
   hipLaunchKernelGGL(causal_attention_kernel, dim3((unsigned)groups), dim3(256), ATT_LDS,
                      static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(q), ld_q,
                      static_cast<const uint16_t*>(k), ld_k, static_cast<const uint16_t*>(v_blk),

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/dynaflow_hip.h"
 
 typedef __bf16 bf16_t;
@@ -16,6 +18,20 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #define DFHIP_DEVICE __device__ __forceinline__
 
 static inline bool dfhip_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Opt a kernel in to `bytes` of dynamic LDS.  The attribute belongs to the (function, device) pair, so `done`
+// - one word per kernel instantiation - carries one bit per device; setting the attribute twice from two
+// threads is harmless, reading a torn flag is not, hence the atomic.
+static inline int dfhip_opt_in_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return DFHIP_ERR_NO_DEVICE;
+  const uint64_t bit = 1ull << (device & 63);
+  if (done.load(std::memory_order_acquire) & bit) return DFHIP_OK;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
+    return DFHIP_ERR_LAUNCH;
+  done.fetch_or(bit, std::memory_order_release);
+  return DFHIP_OK;
+}
 
 static inline int dfhip_check_launch() {
   return hipGetLastError() == hipSuccess ? DFHIP_OK : DFHIP_ERR_LAUNCH;

@@ -466,13 +466,8 @@ gemm_fp8_ring_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ 
 
 int launch_fp8_ring(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
                     const float* a_scale, const float* w_scale, int M, int N, int K, hipStream_t stream) {
-  static bool lds_opted_in = false;
-  if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fp8_ring_kernel<false>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, F8_RING_LDS) != hipSuccess)
-      return DFHIP_ERR_LAUNCH;
-    lds_opted_in = true;
-  }
+  static std::atomic<uint64_t> lds_opted_in{0};   // per instantiation, one bit per device
+  if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(gemm_fp8_ring_kernel<false>), F8_RING_LDS, lds_opted_in)) return rc;
   const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
   hipLaunchKernelGGL(gemm_fp8_ring_kernel<false>, dim3(tiles_m * tiles_n), dim3(256), F8_RING_LDS, stream,
                      static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(W), nullptr,
@@ -484,13 +479,8 @@ int launch_fp8_ring(const void* A, int64_t lda, const void* W, int64_t ldw, void
 int launch_fp8_ring_fused(const void* A, int64_t lda, const void* Wg, const void* Wu, int64_t ldw, void* act,
                           int64_t ld_act, const float* a_scale, const float* wg_scale, const float* wu_scale,
                           float* amax, int M, int I, int K, hipStream_t stream) {
-  static bool lds_opted_in = false;
-  if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fp8_ring_kernel<true>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, F8_RING_LDS) != hipSuccess)
-      return DFHIP_ERR_LAUNCH;
-    lds_opted_in = true;
-  }
+  static std::atomic<uint64_t> lds_opted_in{0};   // per instantiation, one bit per device
+  if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(gemm_fp8_ring_kernel<true>), F8_RING_LDS, lds_opted_in)) return rc;
   const int tiles_m = (M + 255) / 256, tiles_n = (I + 127) / 128;
   hipLaunchKernelGGL(gemm_fp8_ring_kernel<true>, dim3(tiles_m * tiles_n), dim3(256), F8_RING_LDS, stream,
                      static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(Wg), static_cast<const uint8_t*>(Wu),
@@ -675,13 +665,8 @@ gemm_fp8_ring224_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict
 
 int launch_fp8_ring224(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
                        const float* a_scale, const float* w_scale, int M, int N, int K, hipStream_t stream) {
-  static bool lds_opted_in = false;
-  if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fp8_ring224_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, F8_RING_LDS) != hipSuccess)
-      return DFHIP_ERR_LAUNCH;
-    lds_opted_in = true;
-  }
+  static std::atomic<uint64_t> lds_opted_in{0};   // per instantiation, one bit per device
+  if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(gemm_fp8_ring224_kernel), F8_RING_LDS, lds_opted_in)) return rc;
   const int tiles_m = (M + 255) / 256, tiles_n = (N + F8_TBN - 1) / F8_TBN;
   hipLaunchKernelGGL(gemm_fp8_ring224_kernel, dim3(tiles_m * tiles_n), dim3(256), F8_RING_LDS, stream,
                      static_cast<const uint8_t*>(A), static_cast<const uint8_t*>(W), static_cast<uint16_t*>(C),
@@ -701,13 +686,8 @@ int launch_fp8(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, 
                const float* w_scale, int M, int N, int K, hipStream_t stream) {
   constexpr int LDS_BYTES = 2 * (BM + BN) * FROW;
   auto kernel = gemm_fp8_nt_kernel<BM, BN>;
-  static bool lds_opted_in = false;
-  if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            LDS_BYTES) != hipSuccess)
-      return DFHIP_ERR_LAUNCH;
-    lds_opted_in = true;
-  }
+  static std::atomic<uint64_t> lds_opted_in{0};   // per instantiation, one bit per device
+  if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(kernel), LDS_BYTES, lds_opted_in)) return rc;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(256), LDS_BYTES, stream, static_cast<const uint8_t*>(A),
                      static_cast<const uint8_t*>(W), static_cast<uint16_t*>(C), a_scale, w_scale, M, N, K, lda, ldw,

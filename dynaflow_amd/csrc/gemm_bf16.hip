@@ -489,13 +489,8 @@ template <bool FUSED>
 int launch_ring(const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw, void* C, int64_t ldc, int M,
                 int N, int K, int split_k, void* workspace, hipStream_t stream) {
   auto kernel = gemm_bf16_ring_kernel<FUSED>;
-  static bool lds_opted_in = false;   // one flag per instantiation
-  if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            RING_LDS) != hipSuccess)
-      return DFHIP_ERR_LAUNCH;
-    lds_opted_in = true;
-  }
+  static std::atomic<uint64_t> lds_opted_in{0};   // per instantiation, one bit per device
+  if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(kernel), RING_LDS, lds_opted_in)) return rc;
   const int tiles_m = (M + RBM - 1) / RBM;
   const int tiles_n = FUSED ? (N + 127) / 128 : (N + RBN - 1) / RBN;
   int* arrivals = static_cast<int*>(workspace);
@@ -717,13 +712,8 @@ template <bool FUSED, int TN = TBN>
 int launch_ring224(const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw, void* C, int64_t ldc,
                    int M, int N, int K, hipStream_t stream) {
   auto kernel = gemm_bf16_ring224_kernel<FUSED, TN>;
-  static bool lds_opted_in = false;   // one flag per instantiation
-  if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            RING_LDS) != hipSuccess)
-      return DFHIP_ERR_LAUNCH;
-    lds_opted_in = true;
-  }
+  static std::atomic<uint64_t> lds_opted_in{0};   // per instantiation, one bit per device
+  if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(kernel), RING_LDS, lds_opted_in)) return rc;
   constexpr int OUT_N = FUSED ? TN / 2 : TN;
   const int tiles_m = (M + RBM - 1) / RBM;
   const int tiles_n = (N + OUT_N - 1) / OUT_N;
@@ -971,13 +961,8 @@ int launch_skinny(const void* A, int64_t lda, const void* W, const void* W2, int
                   int N, int K, int split_k, void* workspace, hipStream_t stream) {
   if (M > SK_MAX_M || (FUSED && split_k != 1)) return DFHIP_ERR_BAD_SHAPE;
   auto kernel = gemm_bf16_skinny_kernel<FUSED>;
-  static bool lds_opted_in = false;   // one flag per instantiation
-  if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            SK_LDS) != hipSuccess)
-      return DFHIP_ERR_LAUNCH;
-    lds_opted_in = true;
-  }
+  static std::atomic<uint64_t> lds_opted_in{0};   // per instantiation, one bit per device
+  if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(kernel), SK_LDS, lds_opted_in)) return rc;
   constexpr int TILE_N = FUSED ? SK_BN / 2 : SK_BN;
   const int tiles_m = (M + SK_BM - 1) / SK_BM;
   const int tiles_n = (N + TILE_N - 1) / TILE_N;
@@ -996,13 +981,8 @@ int launch(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int6
            int K, hipStream_t stream, const void* R = nullptr) {
   using S = Shape<BM, BN, WAVES_M, WAVES_N>;
   auto kernel = gemm_bf16_nt_kernel<BM, BN, WAVES_M, WAVES_N>;
-  static bool lds_opted_in = false;  // attribute is per function, set once per process
-  if (!lds_opted_in) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            S::LDS_BYTES) != hipSuccess)
-      return DFHIP_ERR_LAUNCH;
-    lds_opted_in = true;
-  }
+  static std::atomic<uint64_t> lds_opted_in{0};   // per instantiation, one bit per device
+  if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(kernel), S::LDS_BYTES, lds_opted_in)) return rc;
   const int tiles_m = (M + BM - 1) / BM;
   const int tiles_n = (N + BN - 1) / BN;
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(S::THREADS), S::LDS_BYTES, stream,
@@ -1172,3 +1152,4 @@ extern "C" int dfhip_gemm_bf16_nt_add(const void* A, int64_t lda, const void* W,
     default: return launch<128, 128, 2, 2>(A, lda, W, ldw, C, ldc, M, N, K, s, R);
   }
 }
+
