@@ -61,6 +61,10 @@ SIGNATURES: dict[str, tuple] = {
         c_int,
         [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, c_int, _P, c_size_t, _P],
     ),
+    "dfhip_gemm_bf16_nt_splitk_static": (
+        c_int,
+        [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, c_int, _P],
+    ),
     "dfhip_gemm_bf16_nt_add": (c_int, [_P, c_int64, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_int, c_int, _P,
                                        c_size_t, _P]),
     "dfhip_gemm_bf16_gate_up_silu": (c_int, [_P, c_int64, _P, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P]),

@@ -17,6 +17,7 @@ extern "C" const char* dfhip_status_string(int status) {
     case DFHIP_ERR_LAUNCH: return "kernel launch failed";
     case DFHIP_ERR_NO_DEVICE: return "no such HIP device";
     case DFHIP_ERR_BAD_ARGUMENT: return "invalid argument";
+    case DFHIP_ERR_TOO_LARGE: return "problem needs more scratch memory than the library holds";
     default: return "unknown status";
   }
 }

@@ -35,7 +35,14 @@
 // gemm_bf16_nt_kernel (generic, register staged, any tile shape of the template)
 //   16-byte global loads into registers while the previous slab multiplies, parked
 //   in two padded LDS buffers, one barrier per slab.  Used for small shapes.
+#include <mutex>
+
 #include "dfhip_common.h"
+
+// Split-K scratch of dfhip_gemm_bf16_nt_splitk_static: arrival counters followed by fp32 partial blocks,
+// laid out like a caller's workspace.  One copy per GPU, held until the process ends.  In host code this
+// name is only a handle for hipGetSymbolAddress; the device address it yields is what launches receive.
+static __device__ __align__(256) unsigned char scratch[DFHIP_SPLITK_STATIC_BYTES];
 
 namespace {
 
@@ -1153,3 +1160,47 @@ extern "C" int dfhip_gemm_bf16_nt_add(const void* A, int64_t lda, const void* W,
   }
 }
 
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[MAX_DEVICES];   // device address of `scratch` on each GPU, looked up on first use
+
+// The address of this GPU's copy of `scratch` (null: the lookup failed).  No allocation happens here.
+void* scratch_on_current_device() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> guard(scratch_mutex);
+  if (!scratch_ptr[device]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    scratch_ptr[device] = p;
+  }
+  return scratch_ptr[device];
+}
+}  // namespace
+
+extern "C" int dfhip_gemm_bf16_nt_splitk_static(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                                                int64_t ldc, int M, int N, int K, int split_k,
+                                                dfhip_stream_t stream) {
+  if (int rc = check_args(A, lda, W, ldw, C, ldc, M, N, K)) return rc;
+  if (split_k < 1 || split_k > 16 || K / BK < split_k) return DFHIP_ERR_BAD_ARGUMENT;
+  const size_t need = dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k);
+  if (need > (size_t)DFHIP_SPLITK_STATIC_BYTES) return DFHIP_ERR_TOO_LARGE;
+  void* ws = nullptr;
+  if (split_k > 1) {
+    ws = scratch_on_current_device();
+    if (!ws) return DFHIP_ERR_NO_DEVICE;
+    // The array keeps what the last call left.  Completed launches leave the counters at zero; they are
+    // cleared all the same (a fill kernel, not a memset node), so that a launch that never finished cannot
+    // poison the next one.  The two split-K kernels size their counter areas differently; the larger one is
+    // cleared (what lies behind the counters are partial blocks, written before they are read).
+    const size_t tiles_ring = (size_t)((M + RBM - 1) / RBM) * ((N + RBN - 1) / RBN);
+    size_t counters = counter_area(tiles_ring);
+    if (M <= SK_MAX_M && skinny_counter_bytes(M, N) > counters) counters = skinny_counter_bytes(M, N);
+    if (int rc = dfhip_fill_u32(ws, 0u, (int64_t)(counters / 4), stream)) return rc;
+  }
+  return dfhip_gemm_bf16_nt_splitk(A, lda, W, ldw, C, ldc, M, N, K, split_k, ws, need, stream);
+}

@@ -42,7 +42,8 @@ typedef enum dfhip_status {
   DFHIP_ERR_BAD_ALIGNMENT = -4, /* pointer or stride not 16-byte aligned */
   DFHIP_ERR_LAUNCH = -5,        /* hipGetLastError() after the launch */
   DFHIP_ERR_NO_DEVICE = -6,
-  DFHIP_ERR_BAD_ARGUMENT = -7
+  DFHIP_ERR_BAD_ARGUMENT = -7,
+  DFHIP_ERR_TOO_LARGE = -8      /* the problem needs more scratch memory than the library holds */
 } dfhip_status;
 
 typedef struct dfhip_device_info {
@@ -114,6 +115,23 @@ size_t dfhip_gemm_bf16_splitk_workspace_bytes(int M, int N, int split_k);
 int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                               int64_t ldc, int M, int N, int K, int split_k, void* workspace,
                               size_t workspace_bytes, dfhip_stream_t stream);
+
+/* dfhip_gemm_bf16_nt_splitk without a workspace argument and without any allocation: the arrival
+ * counters and fp32 partial blocks live in a device array of DFHIP_SPLITK_STATIC_BYTES that is part
+ * of the library's code object (every GPU the library runs on holds its own copy until the process
+ * ends).  It has no counterpart in the reference; it is for callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same
+ * arguments, checks and result bits as dfhip_gemm_bf16_nt_splitk.  A problem whose
+ * dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k) exceeds DFHIP_SPLITK_STATIC_BYTES is refused
+ * with DFHIP_ERR_TOO_LARGE (the limit holds the down projection of a 2048-token nano-batch,
+ * [2048,14336] x [4096,14336]^T with split_k = 2).  All calls on one GPU share the one array: calls
+ * that may overlap in time on a GPU (different streams, different threads) race and must use
+ * dfhip_gemm_bf16_nt_splitk with workspaces of their own.  The counters are cleared by a small fill
+ * kernel ahead of the GEMM on `stream` (no memset node), so the call is legal under capture. */
+#define DFHIP_SPLITK_STATIC_BYTES ((64u << 20) + 4096u)
+int dfhip_gemm_bf16_nt_splitk_static(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                                     int64_t ldc, int M, int N, int K, int split_k,
+                                     dfhip_stream_t stream);
 
 /* C[M,N] = bf16( bf16(A W^T) + R ): the contraction with the residual addition
  * that follows it in a decoder layer (FX nodes linear, add) as the epilogue of the

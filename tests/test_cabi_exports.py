@@ -54,6 +54,11 @@ def test_argument_checks_run_before_any_launch():
     assert lib.dfhip_silu_mul_bf16(16, 8, 16, 8, 16, 8, 1, 7, 0, None) == -2
     assert lib.dfhip_rmsnorm_bf16(16, None, 16, 16, None, 1, 20000, 1e-5, None) == -2
     assert lib.dfhip_gemm_fp8_nt(16, 128, 16, 128, 16, 8, None, None, 1, 8, 128, None) == -1
+    # the split-K entry point with the library's own scratch array refuses what does not fit it
+    assert lib.dfhip_gemm_bf16_nt_splitk_static(16, 4096, 16, 4096, 16, 4096, 4096, 4096, 4096, 2, None) == -8
+    assert lib.dfhip_gemm_bf16_nt_splitk_static(None, 4096, 16, 4096, 16, 4096, 4096, 4096, 4096, 2, None) == -1
+    assert lib.dfhip_gemm_bf16_nt_splitk_static(16, 4096, 16, 4096, 16, 4096, 256, 256, 4096, 17, None) == -7
+    assert b"scratch" in lib.dfhip_status_string(-8)
 
 
 def test_operators_refuse_host_tensors():
