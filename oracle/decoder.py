@@ -63,6 +63,43 @@ def decoder_layer(token_ids, params, seq_len, heads, kv_heads, head_dim, theta=5
     return x + ((g / (1 + torch.exp(-g))) * (h @ P["w_up"].t())) @ P["w_down"].t()
 
 
+def decoder_layer_rows(token_ids, params, rows, seq_len, heads, kv_heads, head_dim, theta=500000.0, eps=1e-5):
+    """decoder_layer(...)[rows] computed without the other rows' share of the work, for sizes where the
+    whole layer takes too long on the CPU: keys and values are needed for every token of a sampled row's
+    sequence (up to the row), queries, the output projection and the MLP only for the sampled rows.
+    Written as one loop over the sampled rows; pinned by equality with decoder_layer on small layers."""
+    P = {k: v.double() for k, v in params.items() if k != "embed"}   # the embedding is gathered first: it is large
+    group = heads // kv_heads
+    half = head_dim // 2
+    freqs = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float64) / head_dim))
+    out = []
+    for r in [int(r) for r in rows]:
+        start, pos = (r // seq_len) * seq_len, r % seq_len
+        x = params["embed"][token_ids[start:start + pos + 1]].double()   # the sequence up to and including the row
+        h = rms_norm(x, P["attn_norm"], eps)
+        ang = torch.arange(pos + 1, dtype=torch.float64)[:, None] * freqs[None, :]
+        rot = torch.polar(torch.ones_like(ang), ang)
+
+        def rotated(t, n):
+            t = t.view(-1, n, head_dim)
+            z = torch.complex(t[..., :half], t[..., half:]) * rot[-t.shape[0]:, None, :]
+            return torch.cat((z.real, z.imag), dim=-1)
+
+        q = rotated(h[-1:] @ P["wq"].t(), heads)[0]                  # [heads, d], position pos
+        k = rotated(h @ P["wk"].t(), kv_heads)                       # [pos+1, kv_heads, d]
+        v = (h @ P["wv"].t()).view(-1, kv_heads, head_dim)
+        a = torch.empty(heads, head_dim, dtype=torch.float64)
+        for hd in range(heads):
+            kv = hd // group
+            p = torch.softmax((k[:, kv, :] @ q[hd]) / math.sqrt(head_dim), dim=0)
+            a[hd] = p @ v[:, kv, :]
+        y = x[-1] + a.reshape(-1) @ P["wo"].t()
+        hm = rms_norm(y, P["mlp_norm"], eps)
+        g = hm @ P["w_gate"].t()
+        out.append(y + ((g / (1 + torch.exp(-g))) * (hm @ P["w_up"].t())) @ P["w_down"].t())
+    return torch.stack(out)
+
+
 def params_of(layer):
     """Collect the parameters of a dynaflow_amd.decoder.DecoderLayer under the names used above."""
     return {

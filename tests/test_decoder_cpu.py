@@ -56,6 +56,18 @@ def test_product_module_matches_oracle_float64():
     assert (got - want).abs().max() / want.abs().max() < 1e-6
 
 
+def test_sampled_row_oracle_equals_the_whole_layer_oracle():
+    """decoder_layer_rows (what the full-size GPU test compares with) against decoder_layer on every row."""
+    layer = small_layer()
+    ids = torch.randint(0, CFG["vocab"], (3 * CFG["seq_len"],), generator=torch.Generator().manual_seed(5))
+    params = ref.params_of(layer)
+    whole = ref.decoder_layer(ids, params, CFG["seq_len"], CFG["heads"], CFG["kv_heads"], CFG["head_dim"])
+    rows = list(range(3 * CFG["seq_len"]))
+    got = ref.decoder_layer_rows(ids, params, rows, CFG["seq_len"], CFG["heads"], CFG["kv_heads"], CFG["head_dim"])
+    assert got.shape == whole.shape
+    assert (got - whole).abs().max() / whole.abs().max() < 1e-12
+
+
 def test_product_rope_matches_oracle():
     cos, sin = rope_tables(12, 16, 500000.0, torch.float64)
     t = torch.randn(2, 12, 3, 16, dtype=torch.float64)

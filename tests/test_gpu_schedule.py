@@ -458,6 +458,96 @@ def test_decoder_layer_attention_beside_mlp_small():
     assert torch.equal(y, y2)
 
 
+def sub_graph_targets(manager):
+    names = [n.target for n in manager.graph_module.graph.nodes if n.op == "call_module"]
+    return names, [[n.target for n in manager.graph_module.__dict__[name].callable_dynamic.graph.nodes
+                    if n.op == "call_function"] for name in names]
+
+
+@pytest.mark.parametrize("batch,S", [(4, 128), (2, 320)])
+def test_decoder_layer_head_dim_128_runs_the_attention_kernel_inside_the_schedule(batch, S):
+    """head_dim 128 (the Llama-3 shape): the attention sub-graph holds the hand-written prefill attention and
+    the paired rotation, fed by column ranges of the stacked q/k/v product, and runs on one stream beside the
+    MLP sub-graph of the other nano-batch.  S = 128 and 320 leave the last 256-row query block ragged."""
+    from dynaflow_amd import ops
+    from oracle import decoder as ref
+
+    shape = dict(hidden=512, heads=4, kv_heads=2, head_dim=128, inter=1408, vocab=1000)
+    manager, compiled, idg, layer, ids = build_decoder(batch, S, **shape)
+    names, (attn_targets, mlp_targets) = sub_graph_targets(manager)
+    assert attn_targets.count(ops.causal_attention) == 1
+    assert attn_targets.count(ops.rope_pair) == 1 and attn_targets.count(ops.rope) == 0
+    assert attn_targets.count(ops.linear_multi) == 1 and attn_targets.count(ops.linear) == 0
+    assert attn_targets.count(ops.linear_add) + attn_targets.count(ops.linear_add_to_output) == 1
+    assert not any(getattr(t, "__name__", "") == "causal_gqa_attention" for t in attn_targets)
+    assert ops.silu_mul in mlp_targets and ops.rms_norm in mlp_targets
+    with torch.no_grad():
+        split = manager.prepare(batch, [S] * batch)
+        y = compiled(idg)
+    torch.cuda.synchronize()
+    assert split.split_indices == [0, (batch // 2) * S, batch * S]
+    assert manager.engine.issue_trace == [(names[0], 0), (names[1], 0), (names[0], 1), (names[1], 1)]
+    want = ref.decoder_layer(ids, ref.params_of(layer), S, 4, 2, 128)
+    assert rel_err(y.float(), want) < TOL["bf16"]
+    # the same kernels issued on one stream give the same bits, and so does a second overlapped run
+    m2, c2, idg2, _, _ = build_decoder(batch, S, serialize=True, **shape)
+    with torch.no_grad():
+        m2.prepare(batch, [S] * batch)
+        y2 = c2(idg2)
+        manager.prepare(batch, [S] * batch)
+        y3 = compiled(idg)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y2) and torch.equal(y, y3)
+
+
+def test_config3_full_size_properties():
+    """The Llama-3-8B decoder layer at its real shape: 8 sequences x 2048 tokens, hidden 4096, 32 query / 8 kv
+    heads of 128, intermediate 14336, vocabulary 128256; two nano-batches of 4 sequences, attention of one beside
+    the MLP of the other.  The float64 oracle takes too long for the whole output at this size, so: (1) sampled
+    (sequence, position) rows against the oracle restricted to those rows, (2) the split schedule against the same
+    layer run as one batch through the same kernels, (3) run-to-run bit identity, (4) serialized == overlapped."""
+    from dynaflow_amd import ops
+    from dynaflow_amd.manager import trivial_split
+    from oracle import decoder as ref
+
+    batch, S = 8, 2048
+    shape = dict(hidden=4096, heads=32, kv_heads=8, head_dim=128, inter=14336, vocab=128256)
+    manager, compiled, idg, layer, ids = build_decoder(batch, S, fuse_silu_epilogue=True, **shape)
+    names, (attn_targets, mlp_targets) = sub_graph_targets(manager)
+    assert attn_targets.count(ops.causal_attention) == 1 and attn_targets.count(ops.rope_pair) == 1
+    with torch.no_grad():
+        split = manager.prepare(batch, [S] * batch)
+        y = compiled(idg)
+    torch.cuda.synchronize()
+    assert split.batch_indices == [0, 4, 8] and split.split_indices == [0, 4 * S, 8 * S]
+    assert manager.engine.issue_trace == [(names[0], 0), (names[1], 0), (names[0], 1), (names[1], 1)]
+    assert bool(torch.isfinite(y.float()).all())
+    # (1) rows of both nano-batches: first and last position of a sequence, the edges of a 256-row query block
+    rows = [0, 255, 2047, 3 * S + 256, 4 * S, 5 * S + 1000, 8 * S - 1]
+    want = ref.decoder_layer_rows(ids, ref.params_of(layer), rows, S, 32, 8, 128)
+    assert rel_err(y[rows].float(), want) < TOL["bf16"]
+    # (2) one batch through the same kernels
+    with torch.no_grad():
+        manager.override_split_config(trivial_split(batch, [S] * batch, False, False))
+        whole = compiled(idg)
+    torch.cuda.synchronize()
+    assert rel_err(y.float(), whole.float()) < 2 ** -6
+    # (3) a second overlapped run has the same bits (no race between the streams)
+    with torch.no_grad():
+        manager.prepare(batch, [S] * batch)
+        y2 = compiled(idg)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y2)
+    # (4) the same launches on one stream
+    del whole, y2
+    m2, c2, idg2, _, _ = build_decoder(batch, S, fuse_silu_epilogue=True, serialize=True, **shape)
+    with torch.no_grad():
+        m2.prepare(batch, [S] * batch)
+        y3 = c2(idg2)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y3)
+
+
 def test_decoder_layer_whole_schedule_graph_with_padded_capture_size():
     """use_cudagraph=True pads the nano-batch sizes to the capture size; the whole-schedule graph
     ignores that padding (it captures the real sizes) and every replay equals the eager run."""
