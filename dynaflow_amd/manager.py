@@ -35,7 +35,8 @@ from dynaflow_amd.config import DynaFlowConfig
 from dynaflow_amd.executor.compiler import SubgraphCompiler
 from dynaflow_amd.interface import ExecutionContext, InputInfo, OpSchedulerBase, SplitConfig
 from dynaflow_amd.matching import split_graph, tag_graph
-from dynaflow_amd.runtime.device import get_device
+from dynaflow_amd.runtime import capture_plan
+from dynaflow_amd.runtime.device import get_device, stream_key
 from dynaflow_amd.runtime.engine import DynaFlowEngine
 
 log = logging.getLogger("dynaflow")
@@ -113,9 +114,6 @@ class _ScheduleGraph:
         self.output = output
 
 
-MAX_WHOLE_GRAPH_SEGMENTS = 2
-
-
 class DynaFlowManager:
     """Splits a traced graph and runs it under a programmable scheduler."""
 
@@ -128,6 +126,8 @@ class DynaFlowManager:
         self.engine: DynaFlowEngine | None = None
         self.graph_dump_path: str | None = None
         self._schedule_graphs: dict[tuple, _ScheduleGraph] = {}
+        #: per captured schedule: "caller" (captured from the caller's side) or "schedule" (from one of its streams)
+        self.capture_origins: dict[tuple, str] = {}
 
     # ------------------------------------------------------------ set-up
     def initialize(
@@ -277,26 +277,6 @@ class DynaFlowManager:
         assert self.config is not None
         assert not kwargs, "whole-schedule graphs take positional graph inputs only"
         assert self.graph_module is not None
-        segments = sum(1 for n in self.graph_module.graph.nodes if n.op == "call_module")
-        if segments > MAX_WHOLE_GRAPH_SEGMENTS:
-            # Ending the stream capture of a six-segment, two-stream schedule crashed inside the runtime
-            # (segmentation fault in the capture's end call); two segments per nano-batch, with up to
-            # four nano-batches, capture and replay correctly.  Until the cause is known the larger
-            # schedules are not captured as one graph: use per-sub-graph graphs or the eager schedule.
-            raise NotImplementedError(
-                f"whole-schedule capture is limited to {MAX_WHOLE_GRAPH_SEGMENTS} sub-graphs per nano-batch "
-                f"(this graph has {segments})"
-            )
-        if self.config.knob("serialize", False) or self.config.knob("streams", "by_kind") != "by_kind":
-            # Schedules in which a nano-batch runs consecutive sub-graphs on ONE stream (the serialized
-            # baseline, one stream per nano-batch) ended the process with a segmentation fault when their
-            # whole-schedule capture was tried (three schedules, once each); what they share, and no capture
-            # that works has, is an event waited for on the stream that recorded it.  No cause has been
-            # shown, so these schedules are not captured as one graph.
-            raise NotImplementedError(
-                "whole-schedule capture is switched off for schedules that keep a nano-batch on one stream "
-                "(serialize, streams=by_nano_batch)"
-            )
         # the whole schedule is captured at its exact size: capture-size padding does not apply
         eager_split = replace(split, use_cudagraph=False, num_tokens_padded=list(split.num_tokens))
         key = (
@@ -305,13 +285,30 @@ class DynaFlowManager:
         )
         entry = self._schedule_graphs.get(key)
         if entry is None:
-            # one eager pass first: lazy one-time set-up (kernel attributes,
-            # allocator growth) must not happen under capture
-            asyncio.run(self._forward_async(args, kwargs, eager_split))
+            # one eager pass first: lazy one-time set-up (kernel attributes, allocator growth) must not
+            # happen under capture; its event log says from which stream the schedule can be captured
+            device = get_device()
+            device.trace = []
+            try:
+                asyncio.run(self._forward_async(args, kwargs, eager_split))
+            finally:
+                event_log, device.trace = device.trace, None
+            caller = stream_key(torch.cuda.current_stream())
+            origin = capture_plan.choose_origin(event_log, caller)
+            if origin is None:
+                raise NotImplementedError(
+                    "this schedule cannot be captured as one graph from any of its streams: streams wait for "
+                    f"each other's events in a cycle {capture_plan.join_cycle(event_log, caller, caller)}; use "
+                    "per-sub-graph graphs (CUDAGraphConfig(enabled=True)) or the eager schedule"
+                )
             torch.cuda.current_stream().synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+            # captured from the caller's side (torch's own capture stream) when that is safe, else from the
+            # stream of the schedule that the others meet at
+            capture_on = {} if origin == caller else {"stream": device.streams_seen[origin]}
+            with torch.cuda.graph(graph, **capture_on):
                 output = asyncio.run(self._forward_async(args, kwargs, eager_split))
+            self.capture_origins[key] = "caller" if origin == caller else "schedule"
             entry = _ScheduleGraph(graph, list(args), self._token_shaped_flags(args), output)
             self._schedule_graphs[key] = entry
         else:

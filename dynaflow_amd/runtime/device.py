@@ -97,13 +97,67 @@ class HostDevice:
         yield
 
 
+def stream_key(stream: "torch.cuda.Stream") -> tuple[int, int]:
+    """What identifies a HIP stream in the event log: (device index, stream handle)."""
+    return (stream.device_index, stream.cuda_stream)
+
+
+class HipEvent:
+    """A HIP event that knows the stream it was recorded on.
+
+    ``wait`` on that very stream issues nothing: stream order already gives the edge, and under stream capture
+    such a wait would make the stream its own child in the runtime's books (see ``capture_plan``).  While the
+    device's ``trace`` is a list, every ``record`` / ``wait`` is logged there in the recording seam's format.
+    """
+
+    __slots__ = ("_owner", "_event", "_recorded_on", "uid")
+    _counter = 0
+
+    def __init__(self, owner: "HipDevice") -> None:
+        HipEvent._counter += 1
+        self.uid = HipEvent._counter
+        self._owner = owner
+        self._event = torch.cuda.Event()
+        self._recorded_on: tuple[int, int] | None = None
+
+    def record(self, stream: "torch.cuda.Stream | None" = None) -> None:
+        stream = stream if stream is not None else torch.cuda.current_stream()
+        self._recorded_on = stream_key(stream)
+        self._owner.note(("record", self.uid, self._recorded_on), stream)
+        self._event.record(stream)
+
+    def wait(self, stream: "torch.cuda.Stream | None" = None) -> None:
+        stream = stream if stream is not None else torch.cuda.current_stream()
+        key = stream_key(stream)
+        self._owner.note(("wait", self.uid, key), stream)
+        if self._recorded_on is None or key == self._recorded_on:
+            return
+        self._event.wait(stream)
+
+    def synchronize(self) -> None:
+        self._event.synchronize()
+
+    def query(self) -> bool:
+        return self._event.query()
+
+
 class HipDevice:
     """The real thing: HIP events, streams and roctx ranges through torch."""
 
     is_gpu = True
 
-    def new_event(self) -> "torch.cuda.Event":
-        return torch.cuda.Event()
+    def __init__(self) -> None:
+        #: while a list: the (kind, event id, stream key) log of every event operation
+        self.trace: list | None = None
+        self.streams_seen: dict[tuple[int, int], "torch.cuda.Stream"] = {}
+
+    def note(self, entry: tuple, stream: "torch.cuda.Stream") -> None:
+        if self.trace is not None:
+            self.trace.append(entry)
+            self.streams_seen[entry[2]] = stream
+
+    def new_event(self) -> HipEvent:
+        return HipEvent(self)
 
     def new_stream(self, name: str | None = None) -> "torch.cuda.Stream":
         return torch.cuda.Stream()

@@ -197,18 +197,6 @@ def compiled_again(manager, compiled, dev, T):
     return out
 
 
-def test_whole_schedule_capture_of_many_sub_graphs_is_refused():
-    """Capturing the whole two-stream schedule of a multi-layer model (more than two sub-graphs per
-    nano-batch) ended in a segmentation fault inside stream capture on this runtime; the manager refuses
-    it instead (per-sub-graph graphs and the eager schedule remain)."""
-    T = 8
-    manager, compiled, dev, *_ = build_decode(T, whole_graph=True, layers=2)
-    with torch.no_grad():
-        manager.prepare(T, [1] * T, use_cudagraph=True)
-        with pytest.raises(NotImplementedError):
-            compiled(*dev)
-
-
 def test_decode_attention_under_graph_capture(ops):
     """The entry points allocate nothing and synchronise nothing, so the operator can be captured into a
     hipGraph: every replay (with eager work between replays) must equal the eager result, and a replay picks
