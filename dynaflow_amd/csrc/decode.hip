@@ -87,7 +87,17 @@ decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
 #pragma unroll
   for (int nb = 0; nb < 8; ++nb) o[nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-  auto step = [&](const KVFrags& f, int c) {
+  auto step = [&](KVFrags& f, int c) {
+    if ((c + 1) * CHUNK > len) {
+      // the last chunk of the sequence: positions from len on may hold anything (a cache that was never
+      // written there, NaN bit patterns included) and their probability 0 would not silence a NaN in the
+      // product, so their V elements are zeroed.  Their K rows need nothing: their scores are replaced below.
+#pragma unroll
+      for (int nb = 0; nb < 8; ++nb)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (c * CHUNK + 8 * g + e >= len) f.v[nb][e] = static_cast<bf16_t>(0.0f);
+    }
     f32x4 s1 = {0.0f, 0.0f, 0.0f, 0.0f}, s2 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {

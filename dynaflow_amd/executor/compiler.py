@@ -80,7 +80,7 @@ class SubgraphBackend:
             if fn is None:
                 handle = get_op_handle()
                 assert isinstance(handle, OperatorHandle) and handle._is_dryrun, (
-                    "Size-specific compilation requires a dry-run with a single OperatorHandle"
+                    "a callable for a listed size is built only inside a dry-run (one operator handle in flight)"
                 )
                 fn = self.callables_per_size[size] = self.compile(list(args), size)
             return fn(*args, **kwargs)

@@ -102,6 +102,9 @@ class OperatorHandle:
     # consumed by the execution backends, not by policies
     _is_dryrun: bool
     _use_cudagraph: bool
+    # which engine issued the handle (not in the reference's record): scratch memory that operators keep per
+    # nano-batch is kept per engine as well, so that two engines never share arrival counters
+    _owner: int = 0
 
 
 class ExecutionContext:

@@ -22,6 +22,7 @@ from __future__ import annotations
 
 import math
 import os
+import weakref
 import threading
 
 import torch
@@ -89,9 +90,9 @@ def _require_device(*tensors: torch.Tensor) -> None:
 
 
 # ---------------------------------------------------------------- linear
-#: split-K workspaces.  Inside a DynaFlow launch: one per (device, nano-batch) - the launches of one nano-batch
-#: are chained one after the other whatever streams they run on, different nano-batches may overlap and must
-#: not share arrival counters.  Outside: one per (device, stream).
+#: split-K workspaces.  Inside a DynaFlow launch: one per (device, engine, nano-batch) - the launches of one
+#: nano-batch are chained one after the other whatever streams they run on; different nano-batches, and the
+#: forwards of different engines, may overlap and must not share arrival counters.  Outside: one per (device, stream).
 _splitk_workspaces: dict[tuple, torch.Tensor] = {}
 #: workspaces that were replaced by larger ones: captured graphs may still point at them
 _retired_workspaces: list[torch.Tensor] = []
@@ -111,7 +112,7 @@ def _zeroed_workspace(cache: dict, device: torch.device, stream: int, nbytes: in
 
     handle = peek_op_handle()
     if isinstance(handle, OperatorHandle):
-        key = (device.index or 0, "nano-batch", handle.batch_idx)
+        key = (device.index or 0, "nano-batch", handle._owner, handle.batch_idx)
     else:
         key = (device.index or 0, "stream", stream)
     ws = cache.get(key)
@@ -233,9 +234,79 @@ torch.library.register_fake("dynaflow_hip::linear_variant", lambda x, w, v: _lin
 
 
 # ------------------------------------------- several projections of one activation
-#: row-wise concatenations of weight groups, keyed by the members' storage and version counters (a weight that
-#: is written to gets a new entry; entries are never dropped, which suits frozen inference weights)
-_stacked_weights: dict[tuple, torch.Tensor] = {}
+class StackedWeightCache:
+    """Row-wise concatenations of weight groups (q / k / v, gate / up), one per group of live weights.
+
+    An entry is keyed by what identifies each member as a tensor in memory - device, address, version counter,
+    shape and row stride - and it lives exactly as long as its members do: every member carries a finalizer that
+    drops the entry, so an address that the allocator hands to a new tensor after a weight was freed never finds
+    the old concatenation.  A member written to in place gets a new version counter and with it a new entry
+    (the stale one is dropped then); pointing ``w.data`` at another tensor changes the address.  The one update
+    no key can see is an in-place write THROUGH ``w.data`` (``w.data.copy_(...)``): callers that update weights
+    that way call ``invalidate()`` (``ops.invalidate_stacked_weights``) afterwards, or switch the stacking off
+    (``stack_projections=False`` at lowering time, or ``enabled = False`` here).
+    """
+
+    def __init__(self) -> None:
+        self.enabled = os.environ.get("DYNAFLOW_STACK_WEIGHTS", "1") != "0"
+        self._entries: dict[tuple, torch.Tensor] = {}
+        self._keys_of_member: dict[int, set] = {}       # id(member) -> keys of the entries it belongs to
+
+    @staticmethod
+    def key_of(weights) -> tuple:
+        return tuple((str(w.device), w.data_ptr(), w._version, tuple(w.shape), w.stride(0)) for w in weights)
+
+    def __len__(self) -> int:
+        return len(self._entries)
+
+    def _drop_member(self, member_id: int) -> None:
+        for key in self._keys_of_member.pop(member_id, ()):
+            self._entries.pop(key, None)
+
+    def get(self, weights, build):
+        """The concatenation for ``weights``; ``build()`` makes it when there is none (it may return None: no
+        entry is kept then)."""
+        key = self.key_of(weights)
+        stacked = self._entries.get(key)
+        if stacked is not None:
+            return stacked
+        stacked = build()
+        if stacked is None:
+            return None
+        for w in weights:
+            known = self._keys_of_member.get(id(w))
+            if known is None:
+                known = self._keys_of_member[id(w)] = set()
+                weakref.finalize(w, self._drop_member, id(w))
+            else:
+                # the same tensor with another address or version: its older concatenations are stale
+                for old in [k for k in known if k != key]:
+                    self._entries.pop(old, None)
+                    known.discard(old)
+            known.add(key)
+        self._entries[key] = stacked
+        return stacked
+
+    def invalidate(self, weights=None) -> None:
+        """Drop every entry (``weights`` None) or the entries that any of ``weights`` belongs to."""
+        if weights is None:
+            self._entries.clear()
+            for known in self._keys_of_member.values():
+                known.clear()
+            return
+        for w in weights:
+            for key in list(self._keys_of_member.get(id(w), ())):
+                self._entries.pop(key, None)
+                self._keys_of_member[id(w)].discard(key)
+
+
+_stacked_weights = StackedWeightCache()
+
+
+def invalidate_stacked_weights(weights=None) -> None:
+    """Forget the stacked copies of weight groups: all of them, or those that any of ``weights`` belongs to.
+    To be called after weights were overwritten in place through ``.data`` (the one update the cache cannot see)."""
+    _stacked_weights.invalidate(weights)
 
 
 def _linear_multi_impl(x: torch.Tensor, weights: list[torch.Tensor]) -> list[torch.Tensor]:
@@ -246,13 +317,14 @@ def _linear_multi_impl(x: torch.Tensor, weights: list[torch.Tensor]) -> list[tor
     if x.dtype != torch.bfloat16 or any(w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] != x.shape[-1]
                                          or w.shape[0] % 8 for w in weights):
         raise RuntimeError("linear_multi: bf16 activation and [N_i, K] bf16 weights with N_i % 8 == 0 expected")
-    key = tuple((w.data_ptr(), w._version, w.shape[0]) for w in weights)
-    stacked = _stacked_weights.get(key)
-    if stacked is None:
+    def build():
         if torch.cuda.is_current_stream_capturing():
-            return [_linear_impl(x, w) for w in weights]      # no allocation that outlives the capture
-        stacked = torch.cat([w.detach() for w in weights], dim=0).contiguous()
-        _stacked_weights[key] = stacked
+            return None                                        # no allocation that outlives the capture
+        return torch.cat([w.detach() for w in weights], dim=0).contiguous()
+
+    stacked = _stacked_weights.get(weights, build) if _stacked_weights.enabled else None
+    if stacked is None:
+        return [_linear_impl(x, w) for w in weights]
     out = _linear_impl(x, stacked)
     parts, first = [], 0
     for w in weights:

@@ -232,6 +232,7 @@ class DynaFlowEngine:
             tag=module.tag,
             _is_dryrun=split_config.is_dryrun,
             _use_cudagraph=split_config.use_cudagraph,
+            _owner=id(self),
         )
 
     def _shared_output_for(self, split_config: SplitConfig, device: Any) -> "_SharedOutput | None":
@@ -351,6 +352,7 @@ class DynaFlowEngine:
             tag=set(),
             _is_dryrun=False,
             _use_cudagraph=split_config.use_cudagraph,
+            _owner=id(self),
         )
         with set_op_handle(handle):
             return self.graph_module(*call_args, **kwargs)

@@ -265,7 +265,11 @@ int dfhip_causal_attention_bf16(const void* q, int64_t ld_q, const void* k, int6
  *   over positions 0 .. lengths[t]-1 of the token's slot, query head h reads kv
  *   head h / (q_heads / kv_heads); q_heads / kv_heads <= 16.  Every cached
  *   element is read once: HBM-bound.  A token whose slot is out of range or
- *   whose length is < 1 gets zeros. */
+ *   whose length is < 1 gets zeros.  Cache positions from lengths[t] on are never
+ *   used, whatever they hold (uninitialised memory, NaN patterns).  A length
+ *   beyond `capacity` is the caller's error and is not reported (nothing here
+ *   synchronises): the append leaves the caches untouched and the token attends
+ *   over the `capacity` cached positions, its own key and value not among them. */
 int dfhip_rope_kv_append_bf16(const void* qkv, int64_t ld_qkv, void* q_out, int64_t ld_q, void* k_cache,
                               void* v_cache, const int32_t* slots, const int32_t* lengths,
                               const float* cos_table, const float* sin_table, int T, int q_heads, int kv_heads,

@@ -330,3 +330,60 @@ def test_one_stream_per_nano_batch_policy(host_device):
                         ("submod_1", 1, "side")]
     with pytest.raises(ValueError):
         MLPOverlapScheduler(make_config(2, streams="per_kernel"))
+
+
+def test_listed_sizes_get_their_own_callable_in_a_dry_run(host_device):
+    """``InductorConfig.compile_sizes`` (dynaflow/executor/compiler.py:69-85): a dry-run at a listed size builds
+    that size's callable; scheduled forwards whose nano-batches have that size dispatch to it, other sizes go to
+    the dynamic callable; outside a dry-run an unbuilt listed size is an error."""
+    cfg = make_config(2)
+    cfg.inductor_config.compile_sizes = {48}
+    model, manager, compiled, x = compile_mlp(cfg, tokens=96)
+    backends = [manager.graph_module.__dict__[n.target] for n in manager.graph_module.graph.nodes
+                if n.op == "call_module"]
+    assert all(b.callables_per_size == {} for b in backends)
+
+    # a scheduled forward with nano-batches of the listed size before any dry-run: refused
+    manager.prepare(96, [96])
+    with pytest.raises(AssertionError, match="dry-run"):
+        with torch.no_grad():
+            compiled(x)
+
+    # the dry-run at 48 tokens builds the callable of that size in every sub-graph
+    small = x[:48].clone()
+    manager.prepare(48, [48], is_dryrun=True)
+    with torch.no_grad():
+        dry = compiled(small)
+    torch.testing.assert_close(dry, model(small), rtol=0, atol=0)
+    assert all(sorted(b.callables_per_size) == [48] for b in backends)
+
+    # count the calls each callable gets from now on
+    calls = {"sized": 0, "dynamic": 0}
+    for b in backends:
+        sized, dynamic = b.callables_per_size[48], b.callable_dynamic
+
+        def counted(fn, key):
+            def call(*a, **k):
+                calls[key] += 1
+                return fn(*a, **k)
+            return call
+
+        b.callables_per_size[48] = counted(sized, "sized")
+        b.callable_dynamic = counted(dynamic, "dynamic")
+
+    split = manager.prepare(96, [96])
+    assert split.num_tokens == [48, 48]
+    with torch.no_grad():
+        y = compiled(x)
+    torch.testing.assert_close(y, model(x), rtol=0, atol=0)
+    assert calls == {"sized": 2 * len(backends), "dynamic": 0}
+
+    # another split of the same input: sizes that are not listed use the dynamic callable
+    calls.update(sized=0, dynamic=0)
+    manager.override_split_config(SplitConfig(num_nano_batches=2, batch_sizes=[40, 56], batch_indices=[0, 40, 96],
+                                              num_tokens=[40, 56], num_tokens_padded=[40, 56],
+                                              split_indices=[0, 40, 96], is_dryrun=False, use_cudagraph=False))
+    with torch.no_grad():
+        y = compiled(x)
+    torch.testing.assert_close(y, model(x), rtol=0, atol=0)
+    assert calls == {"sized": 0, "dynamic": 2 * len(backends)}

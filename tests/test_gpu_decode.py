@@ -72,6 +72,36 @@ def test_decode_attention_against_oracle(ops, heads, kv_heads, capacity, lengths
     assert torch.equal(got_k[untouched], k_nat.double().permute(0, 2, 1, 3)[untouched])
 
 
+def test_decode_attention_ignores_what_lies_past_the_length(ops):
+    """Caches are usually allocated uninitialised or hold recycled slots: NaN and Inf patterns in positions
+    from lengths[t] on (keys and values) must not reach the output, and the result is the one a cache with
+    zeros there gives, bit for bit."""
+    from dynaflow_amd.decode import pack_v_cache
+    from dynaflow_amd.decoder import rope_tables
+
+    heads, kv_heads, capacity = 8, 2, 96
+    lengths = [1, 7, 8, 31, 32, 33, 60, 96]
+    T = len(lengths)
+    g = torch.Generator().manual_seed(21)
+    k_nat = torch.randn(T, kv_heads, capacity, D, generator=g).bfloat16()
+    v_nat = torch.randn(T, kv_heads, capacity, D, generator=g).bfloat16()
+    qkv = torch.randn(T, (heads + 2 * kv_heads) * D, generator=g).bfloat16()
+    slots = torch.arange(T, dtype=torch.int32)
+    lens = torch.tensor(lengths, dtype=torch.int32)
+    cos, sin = (t.cuda() for t in rope_tables(capacity, D, 500000.0))
+    outs = []
+    for junk in (0.0, float("nan"), float("inf")):
+        k, v = k_nat.clone(), v_nat.clone()
+        for t, L in enumerate(lengths):
+            k[t, :, L:], v[t, :, L:] = junk, junk
+        out = ops.decode_attention(qkv.cuda(), k.cuda(), pack_v_cache(v).cuda(), slots.cuda(), lens.cuda(), cos, sin,
+                                   heads, kv_heads)
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(out.float()).all()), junk
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
 def test_decode_attention_bad_slot_or_length_is_harmless(ops):
     from dynaflow_amd.decode import pack_v_cache
     from dynaflow_amd.decoder import rope_tables
@@ -266,3 +296,95 @@ def test_decode_schedule_with_sub_graph_replay(streams):
     names = [n.target for n in manager.graph_module.graph.nodes if n.op == "call_module"]
     wrapper = manager.graph_module.__dict__[names[0]].callable_dynamic
     assert sorted(k[:2] for k in wrapper._entries) == [(half, 0), (half, 1)]
+
+
+class _LayerwiseParams(dict):
+    """``oracle.decode.params_of`` one tensor at a time: float64 copies are made when the oracle asks for them
+    and not kept, so that a 32-layer model never sits on the host in float64 as a whole."""
+
+    def __init__(self, model, embed_rows):
+        super().__init__()
+        self.model = model
+        self.embed_rows = embed_rows                # the embedding rows of the sampled tokens, in their order
+
+    def __getitem__(self, name):
+        if name == "embed":
+            return self.embed_rows
+        kind, i = name.rsplit(".", 1)
+        a, m = self.model.attn[int(i)], self.model.mlp[int(i)]
+        t = {"attn_norm": a.norm_weight, "wqkv": a.wqkv, "wo": a.wo, "mlp_norm": m.norm_weight,
+             "w_gate": m.w_gate, "w_up": m.w_up, "w_down": m.w_down}[kind]
+        return t.detach().double().cpu()
+
+
+def test_config4_full_size_properties():
+    """The decode configuration at its real size: 32 Llama-3-8B-shaped layers, 256 single-token queries, 2048
+    cached positions each (~N(0,1)), two nano-batches of 128.  (1) sampled tokens of both nano-batches against
+    the float64 oracle restricted to those tokens (a token's result depends on its own sequence only), (2) the
+    split schedule against the same step as one batch through the same kernels, (3) run-to-run bit identity,
+    (4) the whole split schedule replayed as ONE hipGraph has the bits of the eager schedule."""
+    from dynaflow_amd.backend import make_backend
+    from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
+    from dynaflow_amd.decode import DecodeModel
+    from dynaflow_amd.manager import DynaFlowManager, trivial_split
+
+    layers, seqs, capacity, heads, kv_heads = 32, 256, 2048, 32, 8
+    print("config 4: build the model on the GPU", flush=True)
+    model = DecodeModel(layers=layers, slots=seqs, capacity=capacity, dtype=torch.bfloat16, device="cuda")
+    model.init_weights(0)
+    model.fill_caches(5)
+    gen = torch.Generator().manual_seed(4)
+    ids = torch.randint(0, 128256, (seqs,), generator=gen)
+    slots = torch.randperm(seqs, generator=gen).int()
+    lengths = torch.full((seqs,), capacity, dtype=torch.int32)
+    lengths[::5] = 1777                               # ragged: a last chunk of 17 positions
+    lengths[3::11] = 1
+    sampled = [0, 3, 127, 128, 255]
+    # the sampled sequences' caches as they are before the step, natural layout, float64, on the host
+    rows = slots[sampled].long().cuda()
+    kc, vc = [], []
+    for a in model.attn:
+        k_nat, v_nat = natural(a.k_cache[rows], a.v_cache[rows])
+        kc.append(k_nat)
+        vc.append(v_nat)
+    cfg = DynaFlowConfig("dynaflow_amd.schedulers:DecoderOverlapScheduler", 2, InductorConfig(enabled=True),
+                         CUDAGraphConfig(enabled=False, capture_sizes=[seqs // 2, seqs]),
+                         {"min_nano_split_tokens": 1, "dump_graph": False, "max_tokens": seqs,
+                          "fuse_silu_epilogue": True, "whole_graph": True, "streams": "by_nano_batch"})
+    manager = DynaFlowManager()
+    torch._dynamo.reset()
+    dev = [t.cuda() for t in (ids, slots, lengths)]
+    for t in dev:
+        torch._dynamo.mark_dynamic(t, 0)
+    compiled = torch.compile(model, backend=make_backend(manager, cfg), fullgraph=True)
+    with torch.no_grad():
+        print("config 4: trace and first call", flush=True)
+        manager.prepare(seqs, [1] * seqs)
+        compiled(*dev)
+        print("config 4: eager two-stream step", flush=True)
+        split = manager.prepare(seqs, [1] * seqs, use_cudagraph=False)
+        y = compiled(*dev).clone()
+        torch.cuda.synchronize()
+        assert split.split_indices == [0, 128, 256]
+        assert len(manager.engine.issue_trace) == 2 * 2 * layers
+        assert bool(torch.isfinite(y.float()).all())
+        print("config 4: oracle on sampled tokens", flush=True)
+        params = _LayerwiseParams(model, model.embed.detach()[ids[sampled].cuda()].double().cpu())
+        local = torch.arange(len(sampled))          # token j of the sample: embedding row j, cache slot j
+        want = ref.decode_step(local, local, lengths[sampled], params, kc, vc, heads, kv_heads)
+        assert rel_err(y[sampled].float(), want) < TOL_BF16
+        print("config 4: the step as one batch", flush=True)
+        manager.override_split_config(trivial_split(seqs, [1] * seqs, False, False))
+        whole = compiled(*dev).clone()
+        torch.cuda.synchronize()
+        assert rel_err(y.float(), whole.float()) < 2 ** -5
+        print("config 4: second eager step", flush=True)
+        manager.prepare(seqs, [1] * seqs, use_cudagraph=False)
+        assert torch.equal(compiled(*dev), y)
+        for i in range(3):
+            print(f"config 4: whole-schedule graph, forward {i}", flush=True)
+            manager.prepare(seqs, [1] * seqs, use_cudagraph=True)
+            out = compiled(*dev)
+            torch.cuda.synchronize()
+            assert torch.equal(out, y), f"replay {i}"
+        assert len(manager._schedule_graphs) == 1

@@ -321,6 +321,65 @@ def test_piecewise_graphs_capture_in_dryrun_and_replay():
         assert sorted(k[:2] for k in wrapper._entries) == [(256, 0), (256, 1)]
 
 
+def test_listed_sizes_dispatch_to_their_own_lowered_callable():
+    """``InductorConfig(compile_sizes={256})``: the dry-run at 256 tokens lowers a callable for that size in
+    every sub-graph, the scheduled forward with 2 x 256 tokens dispatches to it (never to the dynamic one), and
+    the result has the bits of the dynamic callable (dynaflow/executor/compiler.py:69-85)."""
+    from dynaflow_amd import ops
+    from dynaflow_amd.backend import make_backend
+    from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
+    from dynaflow_amd.manager import DynaFlowManager
+    from dynaflow_amd.mlp import SwiGLUMLP
+
+    tokens, hidden, inter = 512, 512, 1408
+    x, wg, wu, wd = mlp.make_inputs(tokens, hidden, inter, torch.bfloat16)
+    model = SwiGLUMLP(hidden, inter, dtype=torch.bfloat16, device="cuda")
+    with torch.no_grad():
+        model.gate_proj.weight.copy_(wg)
+        model.up_proj.weight.copy_(wu)
+        model.down_proj.weight.copy_(wd)
+    xg = x.cuda()
+    outputs = {}
+    for sizes in (None, {256}):
+        cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", 2,
+                             InductorConfig(enabled=True, compile_sizes=sizes),
+                             CUDAGraphConfig(enabled=False, capture_sizes=[tokens]),
+                             {"min_nano_split_tokens": 1, "num_nano_batches": 2, "dump_graph": False})
+        manager = DynaFlowManager()
+        torch._dynamo.reset()
+        torch._dynamo.mark_dynamic(xg, 0)
+        compiled = torch.compile(model, backend=make_backend(manager, cfg), fullgraph=True)
+        with torch.no_grad():
+            manager.prepare(tokens, [tokens])
+            compiled(xg)                                    # trace (512 is not a listed size)
+            backends = [manager.graph_module.__dict__[n.target] for n in manager.graph_module.graph.nodes
+                        if n.op == "call_module"]
+            calls = {"sized": 0, "dynamic": 0}
+            if sizes:
+                manager.prepare(256, [256], is_dryrun=True)
+                dry = compiled(xg[:256].contiguous())
+                torch.cuda.synchronize()
+                assert all(sorted(b.callables_per_size) == [256] for b in backends)
+                for b in backends:
+                    sized_targets = [n.target for n in b.callables_per_size[256].graph.nodes
+                                     if n.op == "call_function"]
+                    assert any(t in (ops.linear, ops.linear_to_output, ops.silu_mul) for t in sized_targets)
+                    b.callables_per_size[256] = (lambda fn: lambda *a, **k: (calls.__setitem__(
+                        "sized", calls["sized"] + 1), fn(*a, **k))[1])(b.callables_per_size[256])
+                    b.callable_dynamic = (lambda fn: lambda *a, **k: (calls.__setitem__(
+                        "dynamic", calls["dynamic"] + 1), fn(*a, **k))[1])(b.callable_dynamic)
+            split = manager.prepare(tokens, [tokens])
+            assert split.num_tokens == [256, 256]
+            outputs[bool(sizes)] = compiled(xg).clone()
+            torch.cuda.synchronize()
+            if sizes:
+                assert calls == {"sized": 2 * len(backends), "dynamic": 0}
+                assert torch.equal(dry, outputs[True][:256])
+    assert torch.equal(outputs[False], outputs[True])
+    want = mlp.mlp_fp32_from(x, wg, wu, wd)
+    assert rel_err(outputs[True].float(), want) < TOL["bf16"]
+
+
 def test_fp8_config_full_size_properties():
     """fp8 70B-shaped layer at full size (x[8192,8192], I=28672, 4 x 2048).  The CPU oracle cannot cover
     this size in test time; the kernels are pinned on small shapes, here the schedule is: (1) the scheduled

@@ -125,3 +125,68 @@ def test_decoder_layer_attention_is_lowered_for_head_dim_128():
     torch.compile(layer, backend=backend, fullgraph=True)(ids)
     _, stats = lower_to_hip(captured["gm"])
     assert "causal_attention" not in stats
+
+
+def test_stacked_weight_cache_keys_and_lifetime():
+    """The cache behind ``linear_multi`` on host tensors (the logic has no device part): an entry dies with its
+    weights, so an address that the allocator reuses never finds an old concatenation; an in-place write and a
+    swapped ``.data`` are seen; a write through ``.data`` needs ``invalidate``."""
+    import gc
+
+    from dynaflow_amd.ops import StackedWeightCache
+
+    cache = StackedWeightCache()
+    builds = []
+
+    def stack(ws):
+        def build():
+            builds.append(1)
+            return torch.cat([w.detach() for w in ws], dim=0)
+        return build
+
+    a, b = torch.randn(8, 16), torch.randn(24, 16)
+    s1 = cache.get([a, b], stack([a, b]))
+    assert cache.get([a, b], stack([a, b])) is s1 and len(builds) == 1
+    assert torch.equal(s1, torch.cat([a, b]))
+    # K and the row count are part of the key: a view of the same storage with another shape is another group
+    a_wide = a.view(4, 32)
+    b_wide = b.view(12, 32)
+    assert cache.get([a_wide, b_wide], stack([a_wide, b_wide])).shape == (16, 32) and len(builds) == 2
+
+    # in-place write: new version counter, new entry, the stale one is gone
+    a.mul_(2.0)
+    s2 = cache.get([a, b], stack([a, b]))
+    assert s2 is not s1 and torch.equal(s2[:8], a) and len(cache) == 2
+
+    # .data pointed at another tensor: new address, new entry
+    a.data = torch.ones(8, 16)
+    s3 = cache.get([a, b], stack([a, b]))
+    assert torch.equal(s3[:8], torch.ones(8, 16)) and len(cache) == 2
+
+    # a write THROUGH .data does not touch the version counter: stale until invalidated
+    a.data.copy_(torch.full((8, 16), 3.0))
+    assert cache.get([a, b], stack([a, b])) is s3 and not torch.equal(s3[:8], a)
+    cache.invalidate([a])
+    s4 = cache.get([a, b], stack([a, b]))
+    assert torch.equal(s4[:8], a)
+
+    # entries die with their weights; a new tensor that lands on a freed weight's address starts from nothing
+    address, version = a.data_ptr(), a._version
+    del a, a_wide, s1, s2, s3, s4
+    gc.collect()
+    assert len(cache) == 0
+    reused = None
+    for _ in range(64):                                   # the host allocator usually hands the block straight back
+        t = torch.zeros(8, 16)
+        if t.data_ptr() == address:
+            reused = t
+            break
+    if reused is not None:
+        n = len(builds)
+        s5 = cache.get([reused, b], stack([reused, b]))
+        assert len(builds) == n + 1 and torch.equal(s5[:8], reused)
+
+    # build() may decline (under stream capture): nothing is kept
+    assert cache.get([b], lambda: None) is None and len(cache) == (1 if reused is not None else 0)
+    cache.invalidate()
+    assert len(cache) == 0
