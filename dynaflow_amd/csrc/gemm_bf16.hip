@@ -36,6 +36,7 @@
 //   16-byte global loads into registers while the previous slab multiplies, parked
 //   in two padded LDS buffers, one barrier per slab.  Used for small shapes.
 #include <mutex>
+#include <type_traits>
 
 #include "dfhip_common.h"
 
@@ -217,10 +218,20 @@ gemm_bf16_nt_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
 
 
 // ------------------------------------------------------------------ ring kernel
+// Results leave the ring kernels through non-temporal stores (`nt`): an output row is written once and read by
+// a later kernel, never by this one, so it should not displace the operand slabs that the workgroups of an
+// XCD share through its L2, nor sit there dirty until the end of the launch (measured on the 8B shapes:
+// gate/up/SiLU launch 3 % faster together with the stores spread over the next tile, down projection 2 %).
 constexpr int RBM = 256, RBN = 256, RTHREADS = 256;
 constexpr int UNIT = 32768, NUNITS = 5, RING_LDS = UNIT * NUNITS;
 constexpr int GROUP_M = 4;   // tiles of one XCD are walked in panels of GROUP_M tile rows
 constexpr int EROW = 272;    // padded row of the epilogue staging area (bytes)
+#ifndef SPLITK_LEAD_PERMILLE
+#define SPLITK_LEAD_PERMILLE 940
+#endif
+// Split-K: share of an even K split (in 1/1000) that a part which only leaves its block takes, and the bound
+// of the last part's wait for the others (sleeps of about a microsecond: a second).
+constexpr int SPLITK_SPIN_LIMIT = 1 << 20;
 
 // 16-byte store / load that is coherent across the XCDs (sc1: written through to, and read
 // from, the memory side instead of the XCD-private L2).  Used for split-K partial blocks so
@@ -266,7 +277,7 @@ __global__ void __launch_bounds__(RTHREADS)
 gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
                       const uint16_t* __restrict__ W2, uint16_t* __restrict__ C,
                       int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n,
-                      int split_k, float* __restrict__ partials, int* __restrict__ arrivals) {
+                      int split_k, int lead_slabs, float* __restrict__ partials, int* __restrict__ arrivals) {
   constexpr int TILE_N = FUSED ? 128 : RBN;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -282,9 +293,10 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   const int in_panel = tile % per_panel;
   const int m0 = (first_m + in_panel % rows_in_panel) * RBM;
   const int n0 = (in_panel / rows_in_panel) * TILE_N;
+  // K split: parts 0 .. split_k-2 take lead_slabs slabs each, the last part takes the rest
   const int slabs_total = K / BK;
-  const int slab0 = (int)((int64_t)slabs_total * part / split_k);
-  const int KT = (int)((int64_t)slabs_total * (part + 1) / split_k) - slab0;
+  const int slab0 = part * lead_slabs;
+  const int KT = part == split_k - 1 ? slabs_total - slab0 : lead_slabs;
 
   uint32_t a_off[8], w_off[8];
 #pragma unroll
@@ -392,30 +404,40 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
 #pragma unroll
     for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
 
+  uint32_t* const poison_cell = reinterpret_cast<uint32_t*>(smem + RING_LDS - 16);   // behind the parked blocks
   if (!FUSED && split_k > 1) {
-    // Every part leaves its fp32 block in `partials` and takes a ticket; the part that draws the
-    // last ticket adds all parts up in part order (so the sum does not depend on who came last)
-    // and writes the tile.  Nobody waits for anybody.
-    f32x4* mine = reinterpret_cast<f32x4*>(partials) + ((int64_t)tile * split_k + part) * (64 * RTHREADS) + tid;
+    // Parts 0 .. split_k-2 of a tile leave their fp32 block in `partials`, count themselves in and are
+    // done; the last part waits for that count, adds the blocks to its own accumulators in part order (so the
+    // sum has one order) and writes the tile.  The last part has the highest launch index of its tile and
+    // workgroups start in launch order, so whoever it waits for is already running or finished - and those
+    // never wait for anybody.  It takes a larger share of K than the others: they write their blocks while
+    // it still multiplies.  The wait is bounded; a tile whose parts never arrived is filled with NaN.
+    int* const counter = arrivals + tile;
+    if (part != split_k - 1) {
+      f32x4* mine = reinterpret_cast<f32x4*>(partials) + ((int64_t)tile * split_k + part) * (64 * RTHREADS) + tid;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+      for (int i = 0; i < 8; ++i)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) store_f32x4_device_coherent(mine + (i * 8 + j) * RTHREADS, acc[i][j]);
-    wait_vmcnt<0>();
+        for (int j = 0; j < 8; ++j) store_f32x4_device_coherent(mine + (i * 8 + j) * RTHREADS, acc[i][j]);
+      wait_vmcnt<0>();
+      __syncthreads();
+      if (tid == 0) __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+    if (tid == 0) {
+      int spins = 0;
+      while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < split_k - 1 &&
+             spins < SPLITK_SPIN_LIMIT) {
+        __builtin_amdgcn_s_sleep(16);
+        ++spins;
+      }
+      // OR-ed into every stored pair of bf16 values: all exponent bits and a mantissa bit, i.e. NaN
+      *poison_cell = spins < SPLITK_SPIN_LIMIT ? 0u : 0x7fc07fc0u;
+      __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // counters are left at zero
+    }
     __syncthreads();
-    int* ticket_cell = reinterpret_cast<int*>(smem);
-    if (tid == 0) *ticket_cell = atomicAdd(arrivals + tile, 1);
-    __syncthreads();
-    const int ticket = *ticket_cell;
-    __syncthreads();
-    if (ticket != split_k - 1) return;
-    if (tid == 0) atomicExch(arrivals + tile, 0);
     const f32x4* all = reinterpret_cast<const f32x4*>(partials) + (int64_t)tile * split_k * (64 * RTHREADS) + tid;
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-      for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    for (int p = 0; p < split_k; ++p) {
+    for (int p = 0; p < split_k - 1; ++p) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         f32x4 v[8];
@@ -424,7 +446,10 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
 #pragma unroll
         for (int j = 0; j < 8; ++j) wait_loaded(v[j]);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] += v[j];
+        for (int j = 0; j < 8; ++j) {
+          acc[i][j] += v[j];
+          asm volatile("" : "+a"(acc[i][j]));   // back to its accumulation registers: no copies pile up
+        }
       }
     }
   }
@@ -458,7 +483,7 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
       const int row = id >> 3, c = id & 7;
       const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * FROW_BYTES + c * 16);
       const int m = m_base + row, n = n_base + c * 8;
-      if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+      if (m < M && n < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n));
     }
     return;
   }
@@ -474,6 +499,7 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
       *reinterpret_cast<u32x2*>(park + (i * 16 + frow) * EROW + (j * 16 + fquad * 4) * 2) = v;
     }
   DFHIP_PIN;
+  const uint32_t poison = split_k > 1 ? *poison_cell : 0u;   // NaN pattern if the other parts of the tile never came
   const int m_base = m0 + wave_m * 128, n_base = n0 + wave_n * 128;
 #pragma unroll 4
   for (int p = 0; p < 32; ++p) {
@@ -487,7 +513,9 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = add2_bf16(v[e], r[e]);
       }
-      *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] |= poison;
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n));
     }
   }
 }
@@ -502,13 +530,17 @@ int launch_ring(const void* A, int64_t lda, const void* W, const void* W2, int64
   const int tiles_n = FUSED ? (N + 127) / 128 : (N + RBN - 1) / RBN;
   int* arrivals = static_cast<int*>(workspace);
   float* partials = nullptr;
+  int lead_slabs = K / BK;
   if (split_k > 1) {
     partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + counter_area((size_t)tiles_m * tiles_n));
+    // the parts that only leave a block take a little less than an even share of K (see the kernel)
+    lead_slabs = (int)((int64_t)(K / BK) * SPLITK_LEAD_PERMILLE / (1000 * split_k));
+    if (lead_slabs < 1) lead_slabs = 1;
   }
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * split_k), dim3(RTHREADS), RING_LDS, stream,
                      static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W),
                      static_cast<const uint16_t*>(W2), static_cast<uint16_t*>(C), M, N, K, lda, ldw, ldc, tiles_m,
-                     tiles_n, split_k, partials, arrivals);
+                     tiles_n, split_k, lead_slabs, partials, arrivals);
   return dfhip_check_launch();
 }
 
@@ -525,6 +557,18 @@ constexpr int TBN = 224;
 // The column count is a template parameter: 224 as described, and 128 (4 x 8 blocks per wave, not FUSED) for
 // shapes whose 256 x 256 tiling has at most half as many tiles as the GPU has CUs - 256 x 128 tiles then fill
 // a round without a split along K and its fp32 partial blocks.
+
+// Fused 224-wide tile: which of the tile's 112 outputs the W row at position `pos` (0..111 within the gate or
+// the up part of the W half) belongs to.  MFMA block j = pos / 16 hands lane quad q = (pos % 16) / 4 the four
+// outputs r = pos % 4.  Blocks are paired: (0,1), (2,3), (4,5) cover 32 outputs each, and quad q owns outputs
+// 8q .. 8q+3 of a pair through the even block and 8q+4 .. 8q+7 through the odd one - eight consecutive
+// outputs, one 16-byte store, four lanes a 64-byte run (the size of a write request; with four outputs per lane
+// a tile went out as 32-byte requests, twice as many, and they held up the loads queued behind them).  The
+// seventh block keeps the plain order.
+DFHIP_DEVICE int fused224_output_of(int pos) {
+  const int j = pos >> 4, n = pos & 15;
+  return j < 6 ? 32 * (j >> 1) + 8 * (n >> 2) + 4 * (j & 1) + (n & 3) : pos;
+}
 
 template <bool FUSED, int TN>
 __global__ void __launch_bounds__(RTHREADS)
@@ -566,7 +610,7 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
   for (int t = 0; t < WP; ++t) {
     const int row = (wave * WP + t) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-    int wr = n0 + ((FUSED && row >= OUT_N) ? row - OUT_N : row);
+    int wr = n0 + (FUSED ? fused224_output_of(row >= OUT_N ? row - OUT_N : row) : row);
     wr = wr < N ? wr : N - 1;
     w_off[t] = (uint32_t)((int64_t)(wr - n0) * ldw * 2 + chunk * 16);
   }
@@ -663,25 +707,33 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
 
   if (FUSED) {
     // silu(gate) * up in registers (blocks j and j + 7 hold the two projections of the same outputs) and
-    // 8-byte stores straight from the registers: a lane owns 4 consecutive columns of one row
+    // stores straight from the registers: a lane owns 8 consecutive outputs of one row per pair of blocks
+    // (see fused224_output_of) and 4 of the seventh block
     const int m_first = m0 + wave * 64 + frow;
+    auto product = [&](int i, int j) {
+      float p[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < JB / 2; ++j) {
-        float p[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][e]));
-          const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j + JB / 2][e]));
-          p[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
-        }
-        u32x2 v;
-        v[0] = pack2_bf16(p[0], p[1]);
-        v[1] = pack2_bf16(p[2], p[3]);
-        const int m = m_first + i * 16, n = n0 + j * 16 + fquad * 4;
-        if (m < M && n < N) *reinterpret_cast<u32x2*>(C + (int64_t)m * ldc + n) = v;
+      for (int e = 0; e < 4; ++e) {
+        const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][e]));
+        const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j + JB / 2][e]));
+        p[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
       }
+      return u32x2{pack2_bf16(p[0], p[1]), pack2_bf16(p[2], p[3])};
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m_first + i * 16;
+#pragma unroll
+      for (int pr = 0; pr < 3; ++pr) {
+        const u32x2 even = product(i, 2 * pr), odd = product(i, 2 * pr + 1);
+        const u32x4 v = {even[0], even[1], odd[0], odd[1]};
+        const int n = n0 + pr * 32 + fquad * 8;   // N % 8 == 0: the run is entirely inside or outside
+        if (m < M && n < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n));
+      }
+      const u32x2 v = product(i, 6);
+      const int n = n0 + 96 + fquad * 4;
+      if (m < M && n < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(C + (int64_t)m * ldc + n));
+    }
     return;
   }
   // park 64 rows x 224 columns per wave as bf16, then store whole row pieces
@@ -710,7 +762,7 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = add2_bf16(v[e], r[e]);
       }
-      *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n));
     }
   }
 }
@@ -728,6 +780,330 @@ int launch_ring224(const void* A, int64_t lda, const void* W, const void* W2, in
                      static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W),
                      static_cast<const uint16_t*>(W2), static_cast<uint16_t*>(C), M, N, K, lda, ldw, ldc, tiles_m,
                      tiles_n);
+  return dfhip_check_launch();
+}
+
+
+// ------------------------------------------------------------------ fused 256 x 224 kernel that walks its tiles
+// gate/up projection with the SiLU*mul epilogue, as gemm_bf16_ring224_kernel<true>, with one workgroup per
+// compute unit that walks several tiles (the tiles the same unit would get round by round) and never lets
+// the ring run dry:
+//   * the DMA of a tile's last two iterations fetches the first slabs of the NEXT tile, so a tile starts with
+//     its operands in LDS;
+//   * a tile's results (56 registers of packed bf16 per lane) are stored during the first iterations of the
+//     next tile's K loop, a few store instructions per slab, instead of all at once at the end of a round.
+// The first MFMAs of a tile take a zero addend instead of the accumulator, so nothing is cleared in between.
+// Full tiles only: M % 256 == 0, N % 112 == 0, K / 64 >= WALK_MIN_SLABS.
+#ifndef WALK_STORES_PER_SLAB
+#define WALK_STORES_PER_SLAB 4
+#endif
+constexpr int WALK_STORES = WALK_STORES_PER_SLAB;    // stores behind one slab of the next tile
+constexpr int WALK_PEEL = 16 / WALK_STORES;          // iterations of the next tile that carry stores
+constexpr int WALK_MIN_SLABS = WALK_PEEL + 3;
+
+template <int I, int N, class F>
+DFHIP_DEVICE void static_for(F& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+__global__ void __launch_bounds__(RTHREADS)
+gemm_bf16_gate_up_silu_walk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
+                                   const uint16_t* __restrict__ W2, uint16_t* __restrict__ C,
+                                   int M, int N, int K, int64_t lda, int64_t ldw, int64_t ldc, int tiles_m,
+                                   int tiles_n) {
+  constexpr int TN = TBN, OUT_N = TN / 2, JB = TN / 16, WP = TN / 32, NR = 4 + JB, MQ = 4 * JB;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int KT = K / BK;
+
+  // Tiles of this workgroup: workgroup b runs on XCD b % 8 and is slot b / 8 there; an XCD owns a contiguous
+  // range of tiles (as remap_xcd deals them) and slot s takes tiles s, s + slots, s + 2 slots, ... of it.
+  const int total = tiles_m * tiles_n;
+  const int slots = gridDim.x / 8;
+  const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+  const int share = total / 8, rest = total % 8;
+  const int first_tile = xcd * share + (xcd < rest ? xcd : rest);
+  const int count = share + (xcd < rest ? 1 : 0);
+  const int n_tiles = slot < count ? (count - slot + slots - 1) / slots : 0;
+  if (n_tiles == 0) return;
+
+  const uint8_t* const w_base = reinterpret_cast<const uint8_t*>(wave >= 2 ? W2 : W);
+  const int per_panel = GROUP_M * tiles_n;
+  auto origin = [&](int walk, int& m0, int& n0) {
+    const int tile = first_tile + slot + walk * slots;
+    const int first_m = (tile / per_panel) * GROUP_M;
+    const int rows_in_panel = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+    const int in_panel = tile % per_panel;
+    m0 = (first_m + in_panel % rows_in_panel) * RBM;
+    n0 = (in_panel / rows_in_panel) * OUT_N;
+  };
+
+  // DMA sources: instruction t of a wave fetches rows 8 t .. 8 t + 7 of the wave's share of a half.  The
+  // swizzled chunk a lane fetches depends on t only through its parity, so two per-lane byte offsets per
+  // operand do; the 16 rows between instructions t and t + 2 go into the wave-uniform base.
+  uint32_t a_off[2], w_off[4];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int row = (wave * 8 + t) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    a_off[t] = (uint32_t)((int64_t)row * lda * 2 + chunk * 16);
+  }
+  // W: the rows of a half are dealt to the MFMA blocks by fused224_output_of.  Instructions 0 .. 4 of a wave lie
+  // in paired blocks, where the rows of instruction t are those of instruction t & 1 shifted by a wave-uniform
+  // number of rows; instructions 5 and 6 (the seventh block, for the odd waves) have offsets of their own.
+  auto w_pos = [&](int t) { return ((wave & 1) * WP + t) * 8; };   // first position of instruction t in its part
+  auto w_lane_off = [&](int t) {
+    const int row = (wave * WP + t) * 8 + (lane >> 3);              // row of the W half in LDS
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    return (uint32_t)((int64_t)fused224_output_of(w_pos(t) + (lane >> 3)) * ldw * 2 + chunk * 16);
+  };
+  w_off[0] = w_lane_off(0);
+  w_off[1] = w_lane_off(1);
+  w_off[2] = w_lane_off(5);
+  w_off[3] = w_lane_off(6);
+  const int64_t a_rows16 = 16 * lda * 2;
+  auto dma_a = [&](int t, const uint8_t* slab, int unit) {
+    dma16_base(unit * UNIT + (wave * 8 + t) * 1024, slab + (t >> 1) * a_rows16, a_off[t & 1]);
+  };
+  auto dma_w = [&](int t, const uint8_t* slab, int unit) {
+    if (t < 5) {
+      const int shift = fused224_output_of(w_pos(t)) - fused224_output_of(w_pos(t & 1));
+      dma16_base(unit * UNIT + (wave * WP + t) * 1024, slab + shift * (ldw * 2), w_off[t & 1]);
+    } else {
+      dma16_base(unit * UNIT + (wave * WP + t) * 1024, slab, w_off[t - 3]);
+    }
+  };
+
+  const int frow = lane & 15, fquad = lane >> 4, fswz = (frow >> 1) & 7;
+  int koff[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) koff[ks] = ((4 * ks + fquad) ^ fswz) * 16;
+  const int a_lane = (wave * 64 + frow) * 128, w_lane = frow * 128;
+
+  f32x4 acc[4][JB];       // defined by the first MFMAs of every tile (zero addend)
+  // the finished tile, waiting to be stored: per 16 rows three runs of 8 outputs and one of 4 (fused224_output_of)
+  u32x4 out16[4][3];
+  u32x2 out8[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int j = 0; j < 3; ++j) out16[i][j] = u32x4{0u, 0u, 0u, 0u};
+    out8[i] = u32x2{0u, 0u};
+  }
+
+  int m0, n0;
+  origin(0, m0, n0);
+  const uint8_t* a_cur = reinterpret_cast<const uint8_t*>(A + (int64_t)m0 * lda);
+  const uint8_t* w_cur = w_base + (int64_t)n0 * ldw * 2;
+  // where the slabs behind the end of the current tile come from: the next tile, or (last tile) its own last two
+  const uint8_t* a_nxt = a_cur + (int64_t)(KT - 2) * (BK * 2);
+  const uint8_t* w_nxt = w_cur + (int64_t)(KT - 2) * (BK * 2);
+  if (n_tiles > 1) {
+    int m1, n1;
+    origin(1, m1, n1);
+    a_nxt = reinterpret_cast<const uint8_t*>(A + (int64_t)m1 * lda);
+    w_nxt = w_base + (int64_t)n1 * ldw * 2;
+  }
+  // results: wave-uniform address of the wave's 64 rows of the tile + a 32-bit byte offset per lane
+  uint8_t* c_cur = reinterpret_cast<uint8_t*>(C + ((int64_t)(m0 + wave * 64)) * ldc + n0);
+  uint8_t* c_pend = c_cur;
+  const int64_t c_rows16 = 16 * ldc * 2;
+  const uint32_t c_lane16 = (uint32_t)((frow * ldc + fquad * 8) * 2), c_lane8 = (uint32_t)((frow * ldc + fquad * 4) * 2);
+
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_a(t, a_cur, 0);
+#pragma unroll
+  for (int t = 0; t < WP; ++t) dma_w(t, w_cur, 1);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) dma_a(t, a_cur + BK * 2, 2);
+#pragma unroll
+  for (int t = 0; t < WP; ++t) dma_w(t, w_cur + BK * 2, 3);
+  wait_vmcnt<8 + WP>();   // slab 0 has landed; slab 1 may still be in flight
+  workgroup_barrier();
+
+  bf16x8 fa[2][4], fw[2][JB];
+  auto read_frag = [&](int pos, int ks, int slot_, int unit_a, int unit_w) {
+    const bool is_a = pos == 1 || pos > JB;
+    const int blk = pos <= 1 ? 0 : pos <= JB ? pos - 1 : pos - JB;
+    if (is_a)
+      fa[slot_][blk] = *reinterpret_cast<const bf16x8*>(smem + unit_a * UNIT + a_lane + koff[ks] + blk * 2048);
+    else
+      fw[slot_][blk] = *reinterpret_cast<const bf16x8*>(smem + unit_w * UNIT + w_lane + koff[ks] + blk * 2048);
+  };
+  auto mfma = [&](int q, int slot_) {   // snake order: odd rows walk the W blocks backwards
+    const int i = q / JB, j = (i & 1) ? JB - 1 - q % JB : q % JB;
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fw[slot_][j]), "v"(fa[slot_][i]));
+  };
+  auto mfma_first = [&](int q) {        // first k-step of a tile: zero addend, the old accumulator is dead
+    const int i = q / JB, j = (i & 1) ? JB - 1 - q % JB : q % JB;
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(acc[i][j]) : "v"(fw[0][j]), "v"(fa[0][i]));
+  };
+  auto store_out = [&](int idx) {   // store idx of the 16 of a tile
+    const int i = idx / 4, run = idx % 4;
+    // written out for the addressing mode: uniform base in scalar registers + the lane's 32-bit offset (the
+    // wait states: the base may have come out of a vector register just before, which a memory instruction
+    // may only read five cycles later, and the compiler does not look into this statement)
+    if (run < 3)
+      asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2 nt" ::"v"(c_lane16), "v"(out16[i][run]),
+                   "s"(c_pend + i * c_rows16 + run * 64)
+                   : "memory");
+    else
+      asm volatile("s_nop 4\n\tglobal_store_dwordx2 %0, %1, %2 nt" ::"v"(c_lane8), "v"(out8[i]),
+                   "s"(c_pend + i * c_rows16 + 192)
+                   : "memory");
+  };
+
+  int ua = 0, uw = 1;   // units of the slab being multiplied
+  int ia = 4, iw = 0;   // units that the A and W halves two slabs ahead go to
+  // One iteration = one slab.  FIRST: first slab of a tile (zero addend).  The iteration issues stores
+  // [STORE0, STORE0 + STORES) of the previous tile (if there is one) ahead of the DMA instructions of its second
+  // k-step: memory instructions complete in order, so by the wait of the next iteration - which needs those
+  // DMA pieces anyway - the stores are no younger than what is waited for, and the count of 8 stays exact.
+  bool pending = false;
+  auto iteration = [&](int kt, auto first_c, auto store0_c, auto stores_c) {
+    constexpr bool FIRST = decltype(first_c)::value;
+    constexpr int STORE0 = decltype(store0_c)::value, STORES = decltype(stores_c)::value;
+    constexpr int A0 = NR + 2, AS = (MQ - A0) / 8;
+    const int s2 = kt + 2;
+    const uint8_t* const pa = s2 < KT ? a_cur + (int64_t)s2 * (BK * 2) : a_nxt + (int64_t)(s2 - KT) * (BK * 2);
+    const uint8_t* const pw = s2 < KT ? w_cur + (int64_t)s2 * (BK * 2) : w_nxt + (int64_t)(s2 - KT) * (BK * 2);
+#pragma unroll
+    for (int q = 0; q < MQ; ++q) {
+      if (FIRST) mfma_first(q); else mfma(q, 0);
+      if (q < NR) read_frag(q, 1, 1, ua, uw);
+      else if (q >= A0 && (q - A0) % AS == 0 && (q - A0) / AS < 8) dma_a((q - A0) / AS, pa, ia);
+      DFHIP_PIN;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    wait_vmcnt<8>();
+    workgroup_barrier();
+    int na = ua + 2; if (na >= NUNITS) na -= NUNITS;
+    int nw = uw + 2; if (nw >= NUNITS) nw -= NUNITS;
+    if (STORES > 0 && pending) {
+#pragma unroll
+      for (int t = 0; t < STORES; ++t) store_out(STORE0 + t);
+    }
+    DFHIP_PIN;
+#pragma unroll
+    for (int q = 0; q < MQ; ++q) {
+      mfma(q, 1);
+      if (q < 4 * WP) { if (q % 4 == 0) dma_w(q / 4, pw, iw); }
+      else if (q < 4 * WP + NR) read_frag(q - 4 * WP, 0, 0, na, nw);
+      DFHIP_PIN;
+    }
+    ua = na; uw = nw;
+    ia += 2; if (ia >= NUNITS) ia -= NUNITS;
+    iw += 2; if (iw >= NUNITS) iw -= NUNITS;
+  };
+  using std::integral_constant;
+  auto peeled = [&](auto p_c) {   // iteration p of a tile
+    constexpr int P = decltype(p_c)::value;
+    iteration(P, integral_constant<bool, P == 0>{}, integral_constant<int, P * WALK_STORES>{},
+              integral_constant<int, WALK_STORES>{});
+  };
+
+#pragma unroll
+  for (int pos = 0; pos < NR; ++pos) read_frag(pos, 0, 0, ua, uw);
+  for (int walk = 0; walk < n_tiles; ++walk) {
+    static_for<0, WALK_PEEL>(peeled);
+    for (int kt = WALK_PEEL; kt < KT; ++kt)
+      iteration(kt, integral_constant<bool, false>{}, integral_constant<int, 0>{}, integral_constant<int, 0>{});
+
+    // the tile is complete once the last MFMAs have written their accumulators (the compiler does not know
+    // that they write late: every later use of an accumulator is tied behind the wait states)
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    // silu(gate) * up with the roundings of the separate kernels (blocks j and j + 7 hold the two projections).
+    // The accumulators are read out here, group by group, by written-out moves: left to the compiler, all of
+    // them were copied out ahead of the arithmetic and did not fit.
+    auto product = [&](int i, int j) {
+      float pr[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float ga, ub;
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(ga) : "a"(acc[i][j][e]));
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(ub) : "a"(acc[i][j + JB / 2][e]));
+        const float gt = bf16_bits_to_f32(f32_to_bf16_bits(ga));
+        const float ut = bf16_bits_to_f32(f32_to_bf16_bits(ub));
+        pr[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
+      }
+      const u32x2 packed = {pack2_bf16(pr[0], pr[1]), pack2_bf16(pr[2], pr[3])};
+      DFHIP_PIN;
+      return packed;
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int run = 0; run < 3; ++run) {
+        const u32x2 even = product(i, 2 * run), odd = product(i, 2 * run + 1);
+        out16[i][run] = u32x4{even[0], even[1], odd[0], odd[1]};
+      }
+      out8[i] = product(i, 6);
+    }
+    // the first fragments of the next tile (the last iteration read them too, into registers that the code
+    // above was free to use: read again rather than kept alive through it)
+#pragma unroll
+    for (int pos = 0; pos < NR; ++pos) read_frag(pos, 0, 0, ua, uw);
+    c_pend = c_cur;
+    pending = true;
+    // on to the next tile: its first slabs are in LDS or on their way
+    a_cur = a_nxt;
+    w_cur = w_nxt;
+    if (walk + 1 < n_tiles) {
+      origin(walk + 1, m0, n0);
+      c_cur = reinterpret_cast<uint8_t*>(C + ((int64_t)(m0 + wave * 64)) * ldc + n0);
+    }
+    if (walk + 2 < n_tiles) {
+      int m2, n2;
+      origin(walk + 2, m2, n2);
+      a_nxt = reinterpret_cast<const uint8_t*>(A + (int64_t)m2 * lda);
+      w_nxt = w_base + (int64_t)n2 * ldw * 2;
+    } else {
+      a_nxt = a_cur + (int64_t)(KT - 2) * (BK * 2);
+      w_nxt = w_cur + (int64_t)(KT - 2) * (BK * 2);
+    }
+  }
+  // the last tile has no successor to hide behind
+#pragma unroll
+  for (int idx = 0; idx < 16; ++idx) store_out(idx);
+  wait_vmcnt<0>();   // no DMA may be in flight when the workgroup gives its LDS back
+}
+
+int compute_units_of_current_device() {
+  static std::atomic<int> cached[64];
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 0;
+  int n = cached[device].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
+    cached[device].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+bool walk_kernel_fits(int M, int N, int K) {
+  return M % RBM == 0 && N % (TBN / 2) == 0 && K / BK >= WALK_MIN_SLABS;
+}
+
+int launch_walk(const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw, void* C, int64_t ldc,
+                int M, int N, int K, hipStream_t stream) {
+  auto kernel = gemm_bf16_gate_up_silu_walk_kernel;
+  static std::atomic<uint64_t> lds_opted_in{0};
+  if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(kernel), RING_LDS, lds_opted_in)) return rc;
+  const int tiles_m = M / RBM, tiles_n = N / (TBN / 2);
+  int grid = compute_units_of_current_device() / 8 * 8;   // one workgroup per compute unit, a multiple of the XCDs
+  if (grid < 8) return DFHIP_ERR_NO_DEVICE;
+  const int rounds = (tiles_m * tiles_n + grid - 1) / grid;
+  // no more workgroups than the longest walk needs: an XCD's tiles spread evenly over its slots
+  const int per_xcd = (tiles_m * tiles_n + 7) / 8;
+  const int slots = (per_xcd + rounds - 1) / rounds;
+  if (slots * 8 < grid) grid = slots * 8;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(RTHREADS), RING_LDS, stream, static_cast<const uint16_t*>(A),
+                     static_cast<const uint16_t*>(W), static_cast<const uint16_t*>(W2), static_cast<uint16_t*>(C),
+                     M, N, K, lda, ldw, ldc, tiles_m, tiles_n);
   return dfhip_check_launch();
 }
 
@@ -922,7 +1298,7 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
       const int row = id >> 2, c = id & 3;
       const u32x4 v = *reinterpret_cast<const u32x4*>(fpark + row * FROW + c * 16);
       const int m = fm_base + row, n = fn_base + c * 8;
-      if (m < M && n < N) *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+      if (m < M && n < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n));
     }
     return;
   }
@@ -955,7 +1331,7 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = add2_bf16(v[e], r[e]);
       }
-      *reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n) = v;
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n));
     }
   }
 }
@@ -1128,8 +1504,12 @@ extern "C" int dfhip_gemm_bf16_gate_up_silu(const void* A, int64_t lda, const vo
   if (M <= 2 * SK_BM && I >= 1024 && K >= 1024)   // decode-sized activations: stream both weights once
     return launch_skinny<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, 1, nullptr,
                                static_cast<hipStream_t>(stream));
-  if (round_fill(M, I, TBN / 2) > round_fill(M, I, 128) + 0.05)
+  if (round_fill(M, I, TBN / 2) > round_fill(M, I, 128) + 0.05) {
+    // more than one round of tiles: workgroups that walk their tiles hide a tile's stores behind the next one
+    if (walk_kernel_fits(M, I, K) && ldo < (1 << 22) && (int64_t)(M / RBM) * (I / (TBN / 2)) > 256)
+      return launch_walk(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, static_cast<hipStream_t>(stream));
     return launch_ring224<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, static_cast<hipStream_t>(stream));
+  }
   return launch_ring<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, 1, nullptr,
                            static_cast<hipStream_t>(stream));
 }

@@ -290,13 +290,17 @@ def test_down_projection_shape_uses_split_k_and_matches_unsplit(ops):
 
 @pytest.mark.parametrize("M,I,K", [(1, 8, 64), (300, 264, 192), (257, 136, 128), (512, 1408, 512),
                                    (2048, 14336, 128), (2000, 14328, 192), (128, 2048, 1024), (100, 1032, 1088),
-                                   (256, 2048, 1024), (200, 1032, 1088)])
+                                   (256, 2048, 1024), (200, 1032, 1088),
+                                   (1024, 8064, 640), (768, 10080, 704), (2048, 14336, 640)])
 def test_gate_up_silu_fused_epilogue(ops, M, I, K):
     """One launch for linear, linear, silu, mul.  The epilogue applies the roundings of the separate kernels,
     so the result has the same bits as linear, linear, silu_mul.  The two large shapes take the 256 x (112
     gate + 112 up) tile (I = 7 * 2^k fills the rounds of 256 workgroups), the others the 256 x (128 + 128)
     tile; (2000, 14328) has ragged tiles in both directions.  The last four (M <= 256) take the weight-streaming
-    kernel with both weights in one 128 x (32 gate + 32 up) x 2 tile, the last two in two row tiles."""
+    kernel with both weights in one 128 x (32 gate + 32 up) x 2 tile, the last two of them in two row tiles.
+    The last three have more full 256 x 112 tiles than the GPU has compute units and at least ten slabs of K:
+    one workgroup per compute unit walks 2 tiles (288 tiles), 1 or 2 (270 tiles in panels of 3 tile rows,
+    unevenly dealt to the XCDs) and 4 tiles, storing a tile while it multiplies the next."""
     x = randn((M, K), 41).bfloat16()
     wg = randn((I, K), 42, 0.05).bfloat16()
     wu = randn((I, K), 43, 0.05).bfloat16()
