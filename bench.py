@@ -37,8 +37,9 @@ TOKENS, HIDDEN, INTER, SPLITS = 4096, 4096, 14336, 2
 BF16_MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E
 # HBM-side bytes per launch, measured with hardware counters; the summaries are under profiles/
-GATE_GEMM_TRAFFIC_BYTES = 429.3e6      # fetch 370.6 MB + write 58.7 MB
-GATE_UP_SILU_TRAFFIC_BYTES = 799.3e6   # fetch 740.6 MB + write 58.7 MB
+GATE_GEMM_TRAFFIC_BYTES = 432.9e6      # fetch 369.4 MB + write 63.5 MB
+GATE_UP_SILU_TRAFFIC_BYTES = 845.8e6   # fetch 738.9 MB + write 106.9 MB (non-temporal stores leave in 64-byte pieces:
+                                       # runs that straddle two are counted twice; 58.7 MB of results)
 METRIC = "MLP-layer tokens/s + overlap speedup vs serial, 8B-shape bf16, 1 MI355X"
 
 
@@ -53,6 +54,8 @@ def parse_args():
     p.add_argument("--kernels-only", action="store_true",
                    help="run only the single-kernel timing loops plus a 256 MiB device copy (used to calibrate "
                         "FETCH_SIZE / WRITE_SIZE under rocprofv3 --pmc); prints the kernel figures as JSON")
+    p.add_argument("--headline-only", action="store_true",
+                   help="only the headline mode (fused epilogue, two streams, one hipGraph): for kernel traces of the step")
     p.add_argument("--fp8", action="store_true",
                    help="measure the fp8 70B-shaped MLP layer (x[8192,8192], I=28672, 4 nano-batches of 2048) "
                         "instead of the headline bf16 configuration")
@@ -633,6 +636,12 @@ def main() -> int:
         print(json.dumps(single_kernels(torch, ops, x, weights, max(20, args.steps), calibration_copy=True)))
         return 0
 
+    if args.headline_only:
+        m_h, c_h = build_path(torch, x, weights, whole_graph=True, fuse_silu_epilogue=True)
+        ms_h, _ = time_steps(torch, m_h, c_h, x, args.steps, args.warmup, use_graph=True)
+        print(json.dumps({"mode": "overlapped_hipgraph+silu_mul_epilogue", "ms_per_step": ms_h, "steps": args.steps}))
+        return 0
+
     # ---- the ways of issuing the schedule (serialized: every launch on one stream, eagerly and as one graph)
     m_ser, c_ser = build_path(torch, x, weights, serialize=True, whole_graph=True)
     ms_serial, y_serial = time_steps(torch, m_ser, c_ser, x, args.steps, args.warmup, use_graph=False)
@@ -743,7 +752,7 @@ def main() -> int:
     # the dominant kernel of the issue mode that `value` comes from
     if fused_wins:
         result["roofline"] = {
-            "kernel": "gemm_bf16_ring224_kernel<true> (gate and up projection of one nano-batch with the SiLU*mul "
+            "kernel": "gemm_bf16_gate_up_silu_walk_kernel (gate and up projection of one nano-batch with the SiLU*mul "
                       "epilogue: [2048,4096] x 2 x [14336,4096]^T -> act[2048,14336])",
             "bound": "mfma",
             "achieved": 2 * gemm_flops / (ms_gus * 1e-3) / 1e12,

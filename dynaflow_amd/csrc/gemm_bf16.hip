@@ -226,11 +226,7 @@ constexpr int RBM = 256, RBN = 256, RTHREADS = 256;
 constexpr int UNIT = 32768, NUNITS = 5, RING_LDS = UNIT * NUNITS;
 constexpr int GROUP_M = 4;   // tiles of one XCD are walked in panels of GROUP_M tile rows
 constexpr int EROW = 272;    // padded row of the epilogue staging area (bytes)
-#ifndef SPLITK_LEAD_PERMILLE
-#define SPLITK_LEAD_PERMILLE 940
-#endif
-// Split-K: share of an even K split (in 1/1000) that a part which only leaves its block takes, and the bound
-// of the last part's wait for the others (sleeps of about a microsecond: a second).
+// Split-K: the bound of the last part's wait for the others (sleeps of about a microsecond: a second).
 constexpr int SPLITK_SPIN_LIMIT = 1 << 20;
 
 // 16-byte store / load that is coherent across the XCDs (sc1: written through to, and read
@@ -410,8 +406,7 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
     // done; the last part waits for that count, adds the blocks to its own accumulators in part order (so the
     // sum has one order) and writes the tile.  The last part has the highest launch index of its tile and
     // workgroups start in launch order, so whoever it waits for is already running or finished - and those
-    // never wait for anybody.  It takes a larger share of K than the others: they write their blocks while
-    // it still multiplies.  The wait is bounded; a tile whose parts never arrived is filled with NaN.
+    // never wait for anybody.  The wait is bounded; a tile whose parts never arrived is filled with NaN.
     int* const counter = arrivals + tile;
     if (part != split_k - 1) {
       f32x4* mine = reinterpret_cast<f32x4*>(partials) + ((int64_t)tile * split_k + part) * (64 * RTHREADS) + tid;
@@ -533,9 +528,7 @@ int launch_ring(const void* A, int64_t lda, const void* W, const void* W2, int64
   int lead_slabs = K / BK;
   if (split_k > 1) {
     partials = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + counter_area((size_t)tiles_m * tiles_n));
-    // the parts that only leave a block take a little less than an even share of K (see the kernel)
-    lead_slabs = (int)((int64_t)(K / BK) * SPLITK_LEAD_PERMILLE / (1000 * split_k));
-    if (lead_slabs < 1) lead_slabs = 1;
+    lead_slabs = (K / BK) / split_k;   // an even split measured best (a smaller share for the parts that only leave a block did not pay)
   }
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * split_k), dim3(RTHREADS), RING_LDS, stream,
                      static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W),

@@ -75,9 +75,11 @@ class HostDevice:
     def new_event(self) -> HostEvent:
         return HostEvent(self.log)
 
-    def new_stream(self, name: str | None = None) -> HostStream:
+    def new_stream(self, name: str | None = None, cu_mask: "list[int] | None" = None) -> HostStream:
         self._stream_count += 1
-        return HostStream(name or f"stream{self._stream_count}")
+        stream = HostStream(name or f"stream{self._stream_count}")
+        stream.cu_mask = cu_mask
+        return stream
 
     def current_stream(self) -> HostStream:
         return _host_state.current
@@ -141,6 +143,28 @@ class HipEvent:
         return self._event.query()
 
 
+def cu_mask_words(first: int, count: int, total: int) -> list[int]:
+    """Mask words for compute units ``first .. first + count - 1`` of ``total``."""
+    if not (0 <= first and count >= 1 and first + count <= total):
+        raise ValueError(f"compute units {first}..{first + count - 1} of {total}")
+    bits = ((1 << count) - 1) << first
+    return [(bits >> (32 * i)) & 0xFFFFFFFF for i in range((total + 31) // 32)]
+
+
+def _masked_stream(cu_mask: list[int]) -> int:
+    """hipExtStreamCreateWithCUMask through the HIP runtime that torch has loaded; returns the stream handle."""
+    import ctypes
+
+    hip = ctypes.CDLL("libamdhip64.so")
+    words = (ctypes.c_uint32 * len(cu_mask))(*cu_mask)
+    stream = ctypes.c_void_p()
+    torch.cuda.current_stream()   # the device's context exists before the raw call
+    rc = hip.hipExtStreamCreateWithCUMask(ctypes.byref(stream), ctypes.c_uint32(len(cu_mask)), words)
+    if rc != 0 or not stream.value:
+        raise RuntimeError(f"hipExtStreamCreateWithCUMask failed with {rc}")
+    return stream.value
+
+
 class HipDevice:
     """The real thing: HIP events, streams and roctx ranges through torch."""
 
@@ -159,8 +183,13 @@ class HipDevice:
     def new_event(self) -> HipEvent:
         return HipEvent(self)
 
-    def new_stream(self, name: str | None = None) -> "torch.cuda.Stream":
-        return torch.cuda.Stream()
+    def new_stream(self, name: str | None = None, cu_mask: "list[int] | None" = None) -> "torch.cuda.Stream":
+        """A stream at the default priority.  ``cu_mask`` (32-bit words, bit i = compute unit i may run this
+        stream's work) makes it a stream restricted to those compute units - what the reference does with green
+        contexts (examples/ae/up-silu-overlap.cu:236-264).  Such a stream lives until the process ends."""
+        if cu_mask is None:
+            return torch.cuda.Stream()
+        return torch.cuda.ExternalStream(_masked_stream(cu_mask))
 
     def current_stream(self) -> "torch.cuda.Stream":
         return torch.cuda.current_stream()

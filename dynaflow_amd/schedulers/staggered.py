@@ -13,7 +13,7 @@ from __future__ import annotations
 from dynaflow_amd.config import DynaFlowConfig
 from dynaflow_amd.interface import ExecutionContext, InputInfo, OpSchedulerBase, SplitConfig
 from dynaflow_amd.matching import MatchingRule
-from dynaflow_amd.runtime.device import get_device
+from dynaflow_amd.runtime.device import cu_mask_words, get_device
 from dynaflow_amd.schedulers.policies import equal_n_way
 
 
@@ -32,8 +32,16 @@ class StaggeredScheduler(OpSchedulerBase):
         self._tag_rules = dict(tag_rules or {})
         self.side_tag = side_tag
         device = get_device()
-        self.comm_stream = device.new_stream("side")
-        self.comp_stream = device.new_stream("main")
+        # "cu_split": n - the side stream may use compute units 0 .. n-1 only and the main stream the others
+        # (hard partition, the reference's green-context experiment); unset: both streams may use every unit
+        cu_split = config.knob("cu_split", None)
+        if cu_split:
+            total = int(config.knob("compute_units", 256))
+            self.comm_stream = device.new_stream("side", cu_mask_words(0, int(cu_split), total))
+            self.comp_stream = device.new_stream("main", cu_mask_words(int(cu_split), total - int(cu_split), total))
+        else:
+            self.comm_stream = device.new_stream("side")
+            self.comp_stream = device.new_stream("main")
         # "by_kind": tagged sub-graphs on the side stream, the others on the main one (the reference's policies);
         # "by_nano_batch": every nano-batch keeps one stream for its whole chain, so that sub-graphs of the same
         # kind of different nano-batches can run side by side as well (with the staggered order they are one

@@ -232,7 +232,7 @@ def test_kernel_errors_become_exceptions(ops):
 
 @pytest.mark.parametrize("M,N,K,split_k", [(300, 264, 512, 2), (300, 264, 512, 3), (256, 512, 512, 8), (513, 256, 1024, 4)])
 def test_gemm_bf16_split_k_against_c_oracle(ops, M, N, K, split_k):
-    """Split-K through the C ABI: parts leave fp32 blocks in a workspace, the last arriver sums them."""
+    """Split-K through the C ABI: parts leave fp32 blocks in a workspace, the last part of a tile adds them to its own."""
     from dynaflow_amd import _cabi
 
     lib = _cabi.load()
@@ -262,6 +262,35 @@ def test_gemm_bf16_split_k_against_c_oracle(ops, M, N, K, split_k):
                                          ws.data_ptr(), 16, stream) == -7
     assert lib.dfhip_gemm_bf16_nt_splitk(ag.data_ptr(), K, wg.data_ptr(), K, out.data_ptr(), N, M, N, K, 9,
                                          ws.data_ptr(), nbytes, stream) == -7
+
+
+def test_split_k_last_part_gives_up_after_a_bounded_wait(ops):
+    """The last part of a tile waits for the other parts' arrival count.  Forced from the host: the counters
+    start at -5, so the count it waits for is never reached.  Every workgroup still ends (the wait is bounded,
+    about half a second here), the tiles come back as NaN instead of a sum with missing parts, the counters are
+    left at zero, and the next launch with the same workspace is correct."""
+    from dynaflow_amd import _cabi
+
+    lib = _cabi.load()
+    M, N, K, split_k = 300, 264, 512, 2
+    a = randn((M, K), 35).bfloat16().cuda()
+    w = randn((N, K), 36, 0.05).bfloat16().cuda()
+    nbytes = lib.dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k)
+    ws = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    tiles = ((M + 255) // 256) * ((N + 255) // 256)
+    ws[: tiles * 4].view(torch.int32).fill_(-5)
+    stream = torch.cuda.current_stream().cuda_stream
+    out = torch.zeros((M, N), dtype=torch.bfloat16, device="cuda")
+    assert lib.dfhip_gemm_bf16_nt_splitk(a.data_ptr(), K, w.data_ptr(), K, out.data_ptr(), N, M, N, K, split_k,
+                                         ws.data_ptr(), nbytes, stream) == 0
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(out.float()).all())
+    assert int(ws[: tiles * 4].view(torch.int32).abs().sum()) == 0
+    assert lib.dfhip_gemm_bf16_nt_splitk(a.data_ptr(), K, w.data_ptr(), K, out.data_ptr(), N, M, N, K, split_k,
+                                         ws.data_ptr(), nbytes, stream) == 0
+    torch.cuda.synchronize()
+    want = a.float() @ w.float().t()
+    assert rel_err(out.float(), want) < 2 ** -7
 
 
 def test_down_projection_shape_uses_split_k_and_matches_unsplit(ops):
