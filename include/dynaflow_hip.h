@@ -103,9 +103,14 @@ int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* split_k);
 /* Split-K flavour of the fast path for shapes with few output tiles (the down
  * projection: [2048,14336] x [4096,14336]^T has 128 tiles of 256x256 for 256
  * compute units).  Each tile is computed by `split_k` workgroups over disjoint
- * K ranges; every part leaves its fp32 block in `workspace`, the part that
- * arrives last adds the blocks up in part order (deterministic) and writes C.
- * No workgroup waits for another.  `workspace` (device memory, 16-byte aligned,
+ * K ranges.  With the 256x256 ring kernel parts 0 .. split_k-2 leave their fp32
+ * block in `workspace` and count themselves in; the last part - the one with the
+ * highest launch index of its tile, so whoever it waits for was started before
+ * it - waits for that count, adds the blocks to its own sum in part order
+ * (deterministic) and writes C.  The wait is bounded (about a second); a tile
+ * whose parts never arrived is written as NaN.  With the weight-streaming kernel
+ * (variant 6) every part leaves a block and the part that arrives last adds them
+ * up; nobody waits.  `workspace` (device memory, 16-byte aligned,
  * at least dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k) bytes) starts
  * with the per-tile arrival counters, which must be ZERO before the first use
  * and are left zero by every launch; launches that may overlap in time need
