@@ -332,6 +332,26 @@ def test_one_stream_per_nano_batch_policy(host_device):
         MLPOverlapScheduler(make_config(2, streams="per_kernel"))
 
 
+def test_compute_unit_split_gives_the_two_streams_disjoint_masks(host_device):
+    """``cu_split=n``: the side stream gets compute units 0 .. n-1, the main stream the others (the counterpart of
+    the reference's green contexts, examples/ae/up-silu-overlap.cu:236-264); unset, the streams carry no mask."""
+    from dynaflow_amd.runtime.device import cu_mask_words
+
+    assert cu_mask_words(0, 32, 256) == [0xFFFFFFFF, 0, 0, 0, 0, 0, 0, 0]
+    assert cu_mask_words(40, 24, 256) == [0, 0xFFFFFF00, 0, 0, 0, 0, 0, 0]
+    assert cu_mask_words(224, 32, 256)[7] == 0xFFFFFFFF
+    with pytest.raises(ValueError):
+        cu_mask_words(250, 16, 256)
+    plain = MLPOverlapScheduler(make_config(2))
+    assert plain.comm_stream.cu_mask is None and plain.comp_stream.cu_mask is None
+    split = MLPOverlapScheduler(make_config(2, cu_split=48))
+    side, main = split.comm_stream.cu_mask, split.comp_stream.cu_mask
+    assert len(side) == len(main) == 8
+    as_int = lambda words: sum(w << (32 * i) for i, w in enumerate(words))
+    assert as_int(side) == (1 << 48) - 1
+    assert as_int(side) & as_int(main) == 0 and as_int(side) | as_int(main) == (1 << 256) - 1
+
+
 def test_listed_sizes_get_their_own_callable_in_a_dry_run(host_device):
     """``InductorConfig.compile_sizes`` (dynaflow/executor/compiler.py:69-85): a dry-run at a listed size builds
     that size's callable; scheduled forwards whose nano-batches have that size dispatch to it, other sizes go to
