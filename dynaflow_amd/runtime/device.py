@@ -151,11 +151,22 @@ def cu_mask_words(first: int, count: int, total: int) -> list[int]:
     return [(bits >> (32 * i)) & 0xFFFFFFFF for i in range((total + 31) // 32)]
 
 
+def _loaded_hip_runtime() -> str:
+    """Path of the HIP runtime that this process has already mapped (the one torch uses): a second copy loaded by
+    its bare name would be another runtime with streams and contexts of its own."""
+    with open("/proc/self/maps") as maps:
+        for line in maps:
+            path = line.rsplit(" ", 1)[-1].strip()
+            if "libamdhip64.so" in path:
+                return path
+    raise RuntimeError("no HIP runtime is loaded in this process")
+
+
 def _masked_stream(cu_mask: list[int]) -> int:
     """hipExtStreamCreateWithCUMask through the HIP runtime that torch has loaded; returns the stream handle."""
     import ctypes
 
-    hip = ctypes.CDLL("libamdhip64.so")
+    hip = ctypes.CDLL(_loaded_hip_runtime())
     words = (ctypes.c_uint32 * len(cu_mask))(*cu_mask)
     stream = ctypes.c_void_p()
     torch.cuda.current_stream()   # the device's context exists before the raw call
