@@ -106,6 +106,29 @@ def test_config2_full_size_properties():
     assert torch.equal(y, y2)
 
 
+def test_config2_headline_mode_full_size():
+    """The mode that the bench reports, at full size: SiLU*mul as the epilogue of the gate/up GEMM (one workgroup
+    per compute unit walks four tiles of the 2048-token nano-batch), one stream per nano-batch, the whole schedule
+    as one hipGraph.  (1) sampled rows against the oracle, (2) the same bits as the unfused two-stream schedule,
+    (3) every replay of the graph equals the eager issue, with eager work between the replays."""
+    manager, compiled, xg, (x, wg, wu, wd) = build(4096, 4096, 14336, torch.bfloat16, prenorm=True,
+                                                   fuse_silu_epilogue=True, whole_graph=True, streams="by_nano_batch")
+    eager, split = run(manager, compiled, xg, 4096)
+    eager = eager.clone()
+    assert split.split_indices == [0, 2048, 4096]
+    rows = torch.tensor([0, 255, 256, 2047, 2048, 3333, 4095])
+    want = mlp.mlp_fp32_from(x[rows], wg, wu, wd)
+    assert rel_err(eager[rows].float(), want) < TOL["bf16"]
+    plain_manager, plain, xp, _ = build(4096, 4096, 14336, torch.bfloat16, prenorm=True)
+    unfused, _ = run(plain_manager, plain, xp, 4096)
+    assert torch.equal(eager, unfused)
+    for _ in range(3):
+        replay, _ = run(manager, compiled, xg, 4096, use_cudagraph=True)
+        assert torch.equal(replay, eager)
+        again, _ = run(plain_manager, plain, xp, 4096)          # eager work of another manager in between
+        assert torch.equal(again, unfused)
+
+
 def test_nano_batch_outputs_land_in_one_buffer(monkeypatch):
     """The down projection of every nano-batch writes its rows of one output buffer: the forward ends without a
     concatenation, and the result has the bits of the schedule that allocates per nano-batch and concatenates."""
