@@ -291,7 +291,9 @@ def fp8_config(torch, steps, warmup):
     del parts
     results = {}
     for name, knobs in (("serialized", {"serialize": True}), ("overlapped", {"whole_graph": True}),
-                        ("overlapped_fused_gate_up", {"whole_graph": True, "fuse_silu_epilogue": True})):
+                        ("overlapped_fused_gate_up", {"whole_graph": True, "fuse_silu_epilogue": True}),
+                        ("stream_per_nano_batch_fused_gate_up", {"whole_graph": True, "fuse_silu_epilogue": True,
+                                                                 "streams": "by_nano_batch"})):
         # the fused mode: gate, up and SiLU*mul + absmax in ONE GEMM launch, cut in front of the down projection
         layer.fuse_gate_up = bool(knobs.get("fuse_silu_epilogue", False))
         extra = {"min_nano_split_tokens": 64, "num_nano_batches": splits, "dump_graph": False, **EXTRA_KNOBS}
@@ -321,7 +323,9 @@ def fp8_config(torch, steps, warmup):
                 torch.cuda.synchronize()
                 results[f"{name}_{mode}_ms"] = (time.perf_counter() - t0) * 1e3 / steps
     flops = 6.0 * tokens * hidden * inter
-    best = min(results["overlapped_graph_ms"], results["overlapped_fused_gate_up_graph_ms"])
+    best_mode = min(("overlapped_graph_ms", "overlapped_fused_gate_up_graph_ms",
+                     "stream_per_nano_batch_fused_gate_up_graph_ms"), key=lambda m: results[m])
+    best = results[best_mode]
     # the dominant kernel, alone: gate + up + SiLU*mul + absmax of one nano-batch in one launch
     from dynaflow_amd import _cabi, ops
     lib = _cabi.load()
@@ -346,7 +350,9 @@ def fp8_config(torch, steps, warmup):
         "data": "synthetic",
         "config": {"workload": "fp8 70B-shaped SwiGLU MLP layer, x[8192,8192], I=28672, 4 nano-batches of 2048, "
                                "per-tensor activation / per-channel weight scales, bf16 output; the best of "
-                               "the separate gate / up / SiLU*mul launches and the one-launch form is reported"},
+                               "the separate gate / up / SiLU*mul launches and the one-launch form (streams by "
+                               "sub-graph kind or one per nano-batch) is reported",
+                   "issue_mode": best_mode[:-3]},
         "timings": results,
         "layer": {"tflops": flops / (best * 1e-3) / 1e12, "frac_of_fp8_mfma_peak": flops / (best * 1e-3) / 1e12 / 5000.0},
         "roofline": {
