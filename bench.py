@@ -672,11 +672,22 @@ def main() -> int:
     ms_fused_graph, yf_graph = time_steps(torch, m_fo, c_fo, x, args.steps, args.warmup, use_graph=True)
     fused_identical = bool(torch.equal(yf_serial, yf_graph))
     yf_graph = yf_graph.clone()
-    # the same with one stream per nano-batch instead of one per kind of sub-graph: the hand-over between two
-    # dependent kernels then lies on a stream whose other stream has work queued, and costs nothing
+    # the same kernels in the order that issues both nano-batches' launches against the same weights back to back
+    # (gate/up/SiLU of nano-batch 0 and 1, then the two down projections): the second launch of a pair finds most of
+    # the weights in the memory-side cache.  Two ways to get that order: the round-robin schedule (the NanoFlow
+    # order of the reference), or one stream per nano-batch (the second gate/up/SiLU launch is queued while the first
+    # holds the compute units)
     m_fn, c_fn = build_path(torch, x, weights, whole_graph=True, fuse_silu_epilogue=True, streams="by_nano_batch")
     ms_fused_graph_nb, yf_graph_nb = time_steps(torch, m_fn, c_fn, x, args.steps, args.warmup, use_graph=True)
-    fused_identical = fused_identical and bool(torch.equal(yf_serial, yf_graph_nb))
+    m_fr, c_fr = build_path(torch, x, weights, whole_graph=True, fuse_silu_epilogue=True, schedule="round_robin")
+    ms_fused_graph_rr, yf_graph_rr = time_steps(torch, m_fr, c_fr, x, args.steps, args.warmup, use_graph=True)
+    fused_identical = (fused_identical and bool(torch.equal(yf_serial, yf_graph_nb))
+                       and bool(torch.equal(yf_serial, yf_graph_rr)))
+    fused_modes = {"+staggered+streams_by_sub_graph_kind": (ms_fused_graph, m_fo, c_fo),
+                   "+staggered+stream_per_nano_batch": (ms_fused_graph_nb, m_fn, c_fn),
+                   "+round_robin+streams_by_sub_graph_kind": (ms_fused_graph_rr, m_fr, c_fr)}
+    best_fused_mode = min(fused_modes, key=lambda m: fused_modes[m][0])
+    ms_fused_best = fused_modes[best_fused_mode][0]
 
     # ---- for comparison only: the 4096 tokens as ONE batch (no nano-batches, one stream, two launches)
     m_un, c_un = build_path(torch, x, weights, min_nano_split_tokens=1 << 30, fuse_silu_epilogue=True)
@@ -697,9 +708,8 @@ def main() -> int:
     silu_bytes = 3.0 * mb * INTER * 2               # read gate + up, write out
     layer_flops = 6.0 * TOKENS * HIDDEN * INTER
 
-    fused_wins = min(ms_fused_graph, ms_fused_graph_nb) < ms_graph
-    per_nano_batch_wins = fused_wins and ms_fused_graph_nb < ms_fused_graph
-    best_ms = min(ms_graph, ms_fused_graph, ms_fused_graph_nb) if fused_wins else ms_graph
+    fused_wins = ms_fused_best < ms_graph
+    best_ms = ms_fused_best if fused_wins else ms_graph
     result = {
         "metric": METRIC,
         "value": TOKENS / (best_ms * 1e-3),
@@ -717,8 +727,8 @@ def main() -> int:
             "workload": f"Llama-3-8B-shaped SwiGLU MLP layer, x[{TOKENS},{HIDDEN}] bf16 pre-normed, I={INTER}, "
                         f"{SPLITS} nano-batches of {mb}, gate/up GEMM of nano-batch 1 beside SiLU*mul+down of "
                         "nano-batch 0 on two HIP streams, whole schedule replayed as one hipGraph",
-            "issue_mode": "overlapped_hipgraph" + ("+silu_mul_epilogue" if fused_wins else "+silu_mul_kernel")
-                          + ("+stream_per_nano_batch" if per_nano_batch_wins else "+streams_by_sub_graph_kind"),
+            "issue_mode": "overlapped_hipgraph" + ("+silu_mul_epilogue" + best_fused_mode if fused_wins
+                                                   else "+silu_mul_kernel+staggered+streams_by_sub_graph_kind"),
             "device": info["arch_name"],
             "compute_units": info["compute_units"],
         },
@@ -743,6 +753,7 @@ def main() -> int:
             "serialized_graph_ms": ms_fused_serial_graph,
             "overlapped_graph_ms": ms_fused_graph,
             "overlapped_graph_stream_per_nano_batch_ms": ms_fused_graph_nb,
+            "overlapped_graph_round_robin_ms": ms_fused_graph_rr,
             "speedup_graph_vs_serialized": ms_fused_serial / ms_fused_graph,
             "speedup_graph_vs_serialized_gpu_side": ms_fused_serial_gpu / ms_fused_graph,
             "speedup_graph_vs_serialized_graph": ms_fused_serial_graph / ms_fused_graph,
@@ -794,7 +805,7 @@ def main() -> int:
     # ---- the same figures under sustained load (`value` stays the short-loop figure defined above)
     load_s = args.sustain_seconds
     if load_s > 0:
-        m_best, c_best = ((m_fn, c_fn) if per_nano_batch_wins else (m_fo, c_fo)) if fused_wins else (m_ovl, c_ovl)
+        m_best, c_best = fused_modes[best_fused_mode][1:] if fused_wins else (m_ovl, c_ovl)
         ms_sustained = sustained_steps(torch, m_best, c_best, x, args.steps, load_s)
         mb_x = x[:mb]
         with torch.no_grad():
