@@ -46,9 +46,16 @@ DFHIP_DEVICE uint32_t f32_to_bf16_bits(float f) {
   return static_cast<uint32_t>(__builtin_bit_cast(uint16_t, h));
 }
 
+// two values rounded and packed by one v_cvt_pk_bf16_f32 (same rounding as f32_to_bf16_bits, lo in bits 0..15)
 DFHIP_DEVICE uint32_t pack2_bf16(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
+// the two bf16 values of a packed pair, as fp32
+DFHIP_DEVICE float bf16_lo_to_f32(uint32_t pair) { return __uint_as_float(pair << 16); }
+DFHIP_DEVICE float bf16_hi_to_f32(uint32_t pair) { return __uint_as_float(pair & 0xffff0000u); }
 
 // silu(g) = g / (1 + e^-g) on the hardware exponential and reciprocal (a few fp32 ulp; the bf16 paths
 // round the result to 8 bits of mantissa right after).  -inf gives NaN like the exact quotient.

@@ -704,14 +704,15 @@ gemm_bf16_ring224_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
     // (see fused224_output_of) and 4 of the seventh block
     const int m_first = m0 + wave * 64 + frow;
     auto product = [&](int i, int j) {
-      float p[4];
+      u32x2 packed;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][e]));
-        const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j + JB / 2][e]));
-        p[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
+      for (int h = 0; h < 2; ++h) {   // two outputs at a time: every rounding is one packed conversion
+        const uint32_t g2 = pack2_bf16(acc[i][j][2 * h], acc[i][j][2 * h + 1]);
+        const uint32_t u2 = pack2_bf16(acc[i][j + JB / 2][2 * h], acc[i][j + JB / 2][2 * h + 1]);
+        const uint32_t s2 = pack2_bf16(silu_fast(bf16_lo_to_f32(g2)), silu_fast(bf16_hi_to_f32(g2)));
+        packed[h] = pack2_bf16(bf16_lo_to_f32(s2) * bf16_lo_to_f32(u2), bf16_hi_to_f32(s2) * bf16_hi_to_f32(u2));
       }
-      return u32x2{pack2_bf16(p[0], p[1]), pack2_bf16(p[2], p[3])};
+      return packed;
     };
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -1013,17 +1014,19 @@ gemm_bf16_gate_up_silu_walk_kernel(const uint16_t* __restrict__ A, const uint16_
     // The accumulators are read out here, group by group, by written-out moves: left to the compiler, all of
     // them were copied out ahead of the arithmetic and did not fit.
     auto product = [&](int i, int j) {
-      float pr[4];
+      float ga[4], ub[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        float ga, ub;
-        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(ga) : "a"(acc[i][j][e]));
-        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(ub) : "a"(acc[i][j + JB / 2][e]));
-        const float gt = bf16_bits_to_f32(f32_to_bf16_bits(ga));
-        const float ut = bf16_bits_to_f32(f32_to_bf16_bits(ub));
-        pr[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(ga[e]) : "a"(acc[i][j][e]));
+        asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(ub[e]) : "a"(acc[i][j + JB / 2][e]));
       }
-      const u32x2 packed = {pack2_bf16(pr[0], pr[1]), pack2_bf16(pr[2], pr[3])};
+      u32x2 packed;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {   // two outputs at a time: every rounding is one packed conversion
+        const uint32_t g2 = pack2_bf16(ga[2 * h], ga[2 * h + 1]), u2 = pack2_bf16(ub[2 * h], ub[2 * h + 1]);
+        const uint32_t s2 = pack2_bf16(silu_fast(bf16_lo_to_f32(g2)), silu_fast(bf16_hi_to_f32(g2)));
+        packed[h] = pack2_bf16(bf16_lo_to_f32(s2) * bf16_lo_to_f32(u2), bf16_hi_to_f32(s2) * bf16_hi_to_f32(u2));
+      }
       DFHIP_PIN;
       return packed;
     };
