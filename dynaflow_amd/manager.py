@@ -236,13 +236,16 @@ class DynaFlowManager:
         execute_queue: asyncio.Queue = asyncio.Queue()
         context = ExecutionContext(split, op_queue, execute_queue)
 
-        if split.is_dryrun:
-            results, events = self.engine.dryrun(args, kwargs, split)
-        else:
-            (results, events), _ = await asyncio.gather(
-                self.engine.execute(args, kwargs, op_queue, execute_queue, split),
-                self.scheduler.schedule(context),
-            )
+        from dynaflow_amd import ops
+
+        with ops.launch_options(split_k=bool(self.config.knob("split_k", True))):
+            if split.is_dryrun:
+                results, events = self.engine.dryrun(args, kwargs, split)
+            else:
+                (results, events), _ = await asyncio.gather(
+                    self.engine.execute(args, kwargs, op_queue, execute_queue, split),
+                    self.scheduler.schedule(context),
+                )
         # the caller's stream continues only after every nano-batch's last launch
         for event in events:
             event.wait()

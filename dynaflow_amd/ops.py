@@ -21,6 +21,7 @@ dynaflow/runtime/engine.py:381.
 from __future__ import annotations
 
 import math
+import contextlib
 import os
 import weakref
 import threading
@@ -98,6 +99,27 @@ _splitk_workspaces: dict[tuple, torch.Tensor] = {}
 _retired_workspaces: list[torch.Tensor] = []
 #: split K for shapes with too few tiles (DYNAFLOW_SPLIT_K=0 switches it off)
 SPLIT_K_ENABLED = os.environ.get("DYNAFLOW_SPLIT_K", "1") != "0"
+_launch_options = threading.local()
+
+
+@contextlib.contextmanager
+def launch_options(split_k: bool = True):
+    """Options for the launches issued inside the block (set by the manager for a forward, from the knobs of its
+    configuration).  ``split_k=False``: a projection with fewer 256 x 256 tiles than the GPU has compute units runs
+    one workgroup per tile instead of splitting K - right when the schedule runs two such projections side by side
+    (one stream per nano-batch), which fill the compute units together and save the fp32 hand-over."""
+    previous = getattr(_launch_options, "split_k", True)
+    _launch_options.split_k = bool(split_k)
+    try:
+        yield
+    finally:
+        _launch_options.split_k = previous
+
+
+def _split_k_on(variant: int) -> bool:
+    """Whether the planned split of K is used: the option above concerns the 256 x 256 ring kernel (variant 0);
+    the weight-streaming kernel of decode-sized activations always splits."""
+    return SPLIT_K_ENABLED and (variant != 0 or getattr(_launch_options, "split_k", True))
 
 
 def _zeroed_workspace(cache: dict, device: torch.device, stream: int, nbytes: int, clear: int = 65536) -> torch.Tensor:
@@ -196,8 +218,8 @@ def _linear_impl(x: torch.Tensor, weight: torch.Tensor, variant: int = -1, split
                 )
                 _cabi.check("dfhip_gemm_bf16_nt_variant", rc)
             else:
-                _, split_k = _plan_bf16(lib, M, N, K)
-                if split_k > 1 and split_k_allowed and SPLIT_K_ENABLED:
+                planned, split_k = _plan_bf16(lib, M, N, K)
+                if split_k > 1 and split_k_allowed and _split_k_on(planned):
                     stream = _stream()
                     nbytes = lib.dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k)
                     ws = _splitk_workspace(x.device, stream, nbytes)
@@ -359,9 +381,9 @@ def _linear_add_impl(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tens
     out = _new_output(M, N, x.dtype, x.device, to_output)
     if M > 0:
         stream = _stream()
-        _, split_k = _plan_bf16(lib, M, N, K)
+        planned, split_k = _plan_bf16(lib, M, N, K)
         ws_ptr, ws_bytes = 0, 0
-        if split_k > 1 and SPLIT_K_ENABLED:
+        if split_k > 1 and _split_k_on(planned):
             nbytes = lib.dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k)
             ws = _splitk_workspace(x.device, stream, nbytes)
             ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()

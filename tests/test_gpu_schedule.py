@@ -129,6 +129,31 @@ def test_config2_headline_mode_full_size():
         assert torch.equal(again, unfused)
 
 
+def test_config2_down_projections_side_by_side_without_k_split():
+    """``split_k=False`` with one stream per nano-batch: each down projection of a 2048-token nano-batch runs one
+    workgroup per 256 x 256 tile (128 of them) instead of two that split K, and the two nano-batches' projections
+    fill the compute units side by side.  Sampled rows against the oracle; the two-stream issue, the one-stream
+    issue and every replay of the whole-schedule graph have the same bits; within a rounding of the split form."""
+    knobs = dict(fuse_silu_epilogue=True, whole_graph=True, streams="by_nano_batch", split_k=False)
+    manager, compiled, xg, (x, wg, wu, wd) = build(4096, 4096, 14336, torch.bfloat16, prenorm=True, **knobs)
+    eager, split = run(manager, compiled, xg, 4096)
+    eager = eager.clone()
+    assert split.split_indices == [0, 2048, 4096]
+    rows = torch.tensor([0, 255, 256, 2047, 2048, 3333, 4095])
+    assert rel_err(eager[rows].float(), mlp.mlp_fp32_from(x[rows], wg, wu, wd)) < TOL["bf16"]
+    for _ in range(3):
+        replay, _ = run(manager, compiled, xg, 4096, use_cudagraph=True)
+        assert torch.equal(replay, eager)
+    serial_manager, serial, xs, _ = build(4096, 4096, 14336, torch.bfloat16, prenorm=True, serialize=True,
+                                          fuse_silu_epilogue=True, split_k=False)
+    one_stream, _ = run(serial_manager, serial, xs, 4096)
+    assert torch.equal(one_stream, eager)
+    split_manager, with_split, xk, _ = build(4096, 4096, 14336, torch.bfloat16, prenorm=True, fuse_silu_epilogue=True)
+    split_form, _ = run(split_manager, with_split, xk, 4096)
+    assert not torch.equal(split_form, eager)            # other order of the fp32 additions ...
+    assert rel_err(split_form.float(), eager.float()) < 2 ** -7   # ... and nothing else
+
+
 def test_nano_batch_outputs_land_in_one_buffer(monkeypatch):
     """The down projection of every nano-batch writes its rows of one output buffer: the forward ends without a
     concatenation, and the result has the bits of the schedule that allocates per nano-batch and concatenates."""

@@ -190,3 +190,25 @@ def test_stacked_weight_cache_keys_and_lifetime():
     assert cache.get([b], lambda: None) is None and len(cache) == (1 if reused is not None else 0)
     cache.invalidate()
     assert len(cache) == 0
+
+
+def test_split_k_option_covers_the_ring_kernel_only():
+    """``launch_options(split_k=False)`` (knob ``split_k``) keeps the 256 x 256 ring kernel (variant 0) from
+    splitting K for the launches issued inside the block; the weight-streaming kernel (variant 6) always splits;
+    the previous setting comes back afterwards, also after an exception."""
+    from dynaflow_amd import ops
+
+    assert ops._split_k_on(0) and ops._split_k_on(6)
+    with ops.launch_options(split_k=False):
+        assert not ops._split_k_on(0)
+        assert ops._split_k_on(6)
+        with ops.launch_options(split_k=True):
+            assert ops._split_k_on(0)
+        assert not ops._split_k_on(0)
+    assert ops._split_k_on(0)
+    try:
+        with ops.launch_options(split_k=False):
+            raise RuntimeError("inside")
+    except RuntimeError:
+        pass
+    assert ops._split_k_on(0)
