@@ -56,6 +56,7 @@ SIGNATURES: dict[str, tuple] = {
         [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, c_int, _P],
     ),
     "dfhip_gemm_bf16_plan": (c_int, [c_int, c_int, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
+    "dfhip_gemm_bf16_plan_shared": (c_int, [c_int, c_int, c_int, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
     "dfhip_gemm_bf16_splitk_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "dfhip_gemm_bf16_nt_splitk": (
         c_int,
@@ -68,6 +69,8 @@ SIGNATURES: dict[str, tuple] = {
     "dfhip_gemm_bf16_nt_add": (c_int, [_P, c_int64, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_int, c_int, _P,
                                        c_size_t, _P]),
     "dfhip_gemm_bf16_gate_up_silu": (c_int, [_P, c_int64, _P, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P]),
+    "dfhip_gemm_bf16_gate_up_silu_shared": (c_int, [_P, c_int64, _P, _P, c_int64, _P, c_int64, c_int, c_int, c_int,
+                                                    c_int, _P]),
     "dfhip_gemm_f32_nt": (c_int, [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, _P]),
     "dfhip_gemm_fp8_nt": (
         c_int,

@@ -1373,10 +1373,11 @@ int launch(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int6
 
 // Fraction of the CU-rounds that do work when [M, N] is cut into 256 x tile_n tiles and the
 // tiles are dealt to 256 CUs in rounds, weighted by the columns of a tile that exist.
-double round_fill(int M, int N, int tile_n) {
-  const int64_t tiles = (int64_t)((M + RBM - 1) / RBM) * ((N + tile_n - 1) / tile_n);
+// `share` launches of this shape run side by side and take their rounds together.
+double round_fill(int M, int N, int tile_n, int share = 1) {
+  const int64_t tiles = (int64_t)((M + RBM - 1) / RBM) * ((N + tile_n - 1) / tile_n) * share;
   const int64_t rounds = (tiles + 255) / 256;
-  return (double)M * N / ((double)rounds * 256 * RBM * tile_n);
+  return (double)M * N * share / ((double)rounds * 256 * RBM * tile_n);
 }
 
 int check_args(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
@@ -1411,8 +1412,13 @@ extern "C" int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void
 }
 
 extern "C" int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* split_k) {
+  return dfhip_gemm_bf16_plan_shared(M, N, K, 1, variant, split_k);
+}
+
+extern "C" int dfhip_gemm_bf16_plan_shared(int M, int N, int K, int share, int* variant, int* split_k) {
   if (!variant || !split_k) return DFHIP_ERR_NULL_POINTER;
   if (M < 1 || N < 1 || K < 1) return DFHIP_ERR_BAD_SHAPE;
+  if (share < 1 || share > 16) return DFHIP_ERR_BAD_ARGUMENT;
   // The 256x256 ring kernel whenever the problem has more than half a tile of rows and columns
   // and enough tiles to occupy a good part of the 256 CUs; the small register-staged tile
   // otherwise.  With at most half as many tiles as CUs, K is split so that every CU gets a part.
@@ -1437,7 +1443,7 @@ extern "C" int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* spli
   }
   if (M > 128 && N > 128 && big_tiles >= 32) {
     *variant = 0;
-    int s = (int)(256 / big_tiles);
+    int s = (int)(256 / (big_tiles * share));   // launches that run side by side fill the compute units together
     if (s > 8) s = 8;
     while (s > 1 && K / BK < 16 * s) --s;   // keep at least 16 slabs per part
     if (s > 1) *split_k = s;
@@ -1449,7 +1455,7 @@ extern "C" int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* spli
       return DFHIP_OK;
     }
     // 256 x 224 tiles when they fill the rounds of 256 workgroups clearly better (N = 7 * 2^k)
-    if (s <= 1 && round_fill(M, N, TBN) > round_fill(M, N, RBN) + 0.05) *variant = 5;
+    if (s <= 1 && round_fill(M, N, TBN, share) > round_fill(M, N, RBN, share) + 0.05) *variant = 5;
   }
   return DFHIP_OK;
 }
@@ -1494,15 +1500,26 @@ extern "C" int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void*
 extern "C" int dfhip_gemm_bf16_gate_up_silu(const void* A, int64_t lda, const void* W_gate, const void* W_up,
                                             int64_t ldw, void* Out, int64_t ldo, int M, int I, int K,
                                             dfhip_stream_t stream) {
+  return dfhip_gemm_bf16_gate_up_silu_shared(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, 1, stream);
+}
+
+extern "C" int dfhip_gemm_bf16_gate_up_silu_shared(const void* A, int64_t lda, const void* W_gate, const void* W_up,
+                                                   int64_t ldw, void* Out, int64_t ldo, int M, int I, int K,
+                                                   int share, dfhip_stream_t stream) {
   if (!W_up) return DFHIP_ERR_NULL_POINTER;
+  if (share < 1 || share > 16) return DFHIP_ERR_BAD_ARGUMENT;
   if (int rc = check_args(A, lda, W_gate, ldw, Out, ldo, M, I, K)) return rc;
   if (!dfhip_aligned16(W_up)) return DFHIP_ERR_BAD_ALIGNMENT;
   if (M <= 2 * SK_BM && I >= 1024 && K >= 1024)   // decode-sized activations: stream both weights once
     return launch_skinny<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, 1, nullptr,
                                static_cast<hipStream_t>(stream));
-  if (round_fill(M, I, TBN / 2) > round_fill(M, I, 128) + 0.05) {
-    // more than one round of tiles: workgroups that walk their tiles hide a tile's stores behind the next one
-    if (walk_kernel_fits(M, I, K) && ldo < (1 << 22) && (int64_t)(M / RBM) * (I / (TBN / 2)) > 256)
+  // the 256 x (112 + 112) tile when it fills the rounds of 256 workgroups clearly better than the 256 x (128 + 128)
+  // one, which moves fewer bytes through LDS per flop; launches that run side by side take their rounds together
+  // (two launches of the 8B shape at 2048 rows: 2 x 896 square tiles are exactly 7 rounds)
+  if (round_fill(M, I, TBN / 2, share) > round_fill(M, I, 128, share) + 0.05) {
+    // a launch that has the GPU to itself and more than one round of tiles: workgroups that walk their tiles hide
+    // a tile's stores behind the next one (they hold their compute units to the end, so nothing runs beside them)
+    if (share == 1 && walk_kernel_fits(M, I, K) && ldo < (1 << 22) && (int64_t)(M / RBM) * (I / (TBN / 2)) > 256)
       return launch_walk(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, static_cast<hipStream_t>(stream));
     return launch_ring224<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, static_cast<hipStream_t>(stream));
   }

@@ -238,7 +238,7 @@ class DynaFlowManager:
 
         from dynaflow_amd import ops
 
-        with ops.launch_options(split_k=bool(self.config.knob("split_k", True))):
+        with ops.launch_options(side_by_side=int(self.config.knob("side_by_side", 1))):
             if split.is_dryrun:
                 results, events = self.engine.dryrun(args, kwargs, split)
             else:

@@ -103,23 +103,22 @@ _launch_options = threading.local()
 
 
 @contextlib.contextmanager
-def launch_options(split_k: bool = True):
+def launch_options(side_by_side: int = 1):
     """Options for the launches issued inside the block (set by the manager for a forward, from the knobs of its
-    configuration).  ``split_k=False``: a projection with fewer 256 x 256 tiles than the GPU has compute units runs
-    one workgroup per tile instead of splitting K - right when the schedule runs two such projections side by side
-    (one stream per nano-batch), which fill the compute units together and save the fp32 hand-over."""
-    previous = getattr(_launch_options, "split_k", True)
-    _launch_options.split_k = bool(split_k)
+    configuration).  ``side_by_side=n``: the schedule runs the same sub-graph of ``n`` nano-batches at the same time
+    (one stream per nano-batch), so a bf16 GEMM shares the compute units with ``n - 1`` launches of its own shape:
+    the kernel plan takes their tiles together - K is split less or not at all, and the tile shape is chosen for
+    the rounds that the launches fill together."""
+    previous = getattr(_launch_options, "side_by_side", 1)
+    _launch_options.side_by_side = max(1, int(side_by_side))
     try:
         yield
     finally:
-        _launch_options.split_k = previous
+        _launch_options.side_by_side = previous
 
 
-def _split_k_on(variant: int) -> bool:
-    """Whether the planned split of K is used: the option above concerns the 256 x 256 ring kernel (variant 0);
-    the weight-streaming kernel of decode-sized activations always splits."""
-    return SPLIT_K_ENABLED and (variant != 0 or getattr(_launch_options, "split_k", True))
+def _side_by_side() -> int:
+    return getattr(_launch_options, "side_by_side", 1)
 
 
 def _zeroed_workspace(cache: dict, device: torch.device, stream: int, nbytes: int, clear: int = 65536) -> torch.Tensor:
@@ -159,19 +158,15 @@ def _splitk_workspace(device: torch.device, stream: int, nbytes: int) -> torch.T
 
 
 def _plan_bf16(lib, M: int, N: int, K: int) -> tuple[int, int]:
+    """(kernel variant, split of K) for a bf16 GEMM, for as many launches side by side as the forward declared."""
     import ctypes
 
     variant, split_k = ctypes.c_int(0), ctypes.c_int(1)
-    _cabi.check("dfhip_gemm_bf16_plan", lib.dfhip_gemm_bf16_plan(M, N, K, ctypes.byref(variant), ctypes.byref(split_k)))
+    _cabi.check("dfhip_gemm_bf16_plan_shared", lib.dfhip_gemm_bf16_plan_shared(
+        M, N, K, _side_by_side(), ctypes.byref(variant), ctypes.byref(split_k)))
     return variant.value, split_k.value
 
 
-# ------------------------------------------------------------ output rows
-# The engine may offer, for the sub-graph call that produces a nano-batch's share of the model output, the rows
-# of ONE buffer shared by all nano-batches; the ``*_to_output`` operators (what the lowering makes of the
-# projection whose result the sub-graph returns) write there, and the per-nano-batch results then need no
-# concatenation.  An offer holds for one operator call of the offering thread and is withdrawn by the engine
-# after the sub-graph call.
 _output_offer = threading.local()
 
 
@@ -219,7 +214,7 @@ def _linear_impl(x: torch.Tensor, weight: torch.Tensor, variant: int = -1, split
                 _cabi.check("dfhip_gemm_bf16_nt_variant", rc)
             else:
                 planned, split_k = _plan_bf16(lib, M, N, K)
-                if split_k > 1 and split_k_allowed and _split_k_on(planned):
+                if split_k > 1 and split_k_allowed and SPLIT_K_ENABLED:
                     stream = _stream()
                     nbytes = lib.dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k)
                     ws = _splitk_workspace(x.device, stream, nbytes)
@@ -228,6 +223,12 @@ def _linear_impl(x: torch.Tensor, weight: torch.Tensor, variant: int = -1, split
                         ws.data_ptr(), ws.numel(), stream,
                     )
                     _cabi.check("dfhip_gemm_bf16_nt_splitk", rc)
+                elif _side_by_side() > 1 and planned != 6:
+                    # the plan for launches side by side, not the one the library makes for a lone launch
+                    rc = lib.dfhip_gemm_bf16_nt_variant(
+                        a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), N, M, N, K, planned, _stream()
+                    )
+                    _cabi.check("dfhip_gemm_bf16_nt_variant", rc)
                 else:
                     rc = lib.dfhip_gemm_bf16_nt(
                         a.data_ptr(), lda, w.data_ptr(), ldw, out.data_ptr(), N, M, N, K, _stream()
@@ -381,9 +382,9 @@ def _linear_add_impl(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tens
     out = _new_output(M, N, x.dtype, x.device, to_output)
     if M > 0:
         stream = _stream()
-        planned, split_k = _plan_bf16(lib, M, N, K)
+        _, split_k = _plan_bf16(lib, M, N, K)
         ws_ptr, ws_bytes = 0, 0
-        if split_k > 1 and _split_k_on(planned):
+        if split_k > 1 and SPLIT_K_ENABLED:
             nbytes = lib.dfhip_gemm_bf16_splitk_workspace_bytes(M, N, split_k)
             ws = _splitk_workspace(x.device, stream, nbytes)
             ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
@@ -420,8 +421,8 @@ def _gate_up_silu_impl(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor
         ldg = K
     out = torch.empty((M, I), dtype=x.dtype, device=x.device)
     if M > 0:
-        rc = lib.dfhip_gemm_bf16_gate_up_silu(
-            a.data_ptr(), lda, wg.data_ptr(), wu.data_ptr(), ldg, out.data_ptr(), I, M, I, K, _stream()
+        rc = lib.dfhip_gemm_bf16_gate_up_silu_shared(
+            a.data_ptr(), lda, wg.data_ptr(), wu.data_ptr(), ldg, out.data_ptr(), I, M, I, K, _side_by_side(), _stream()
         )
         _cabi.check("dfhip_gemm_bf16_gate_up_silu", rc)
     return out.view(*x.shape[:-1], I)

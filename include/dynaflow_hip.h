@@ -99,6 +99,12 @@ int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void* W, int64_
  * the split_k a caller with a workspace should pass to dfhip_gemm_bf16_nt_splitk
  * (1 = no split). */
 int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* split_k);
+/* The same choice for a launch that runs side by side with `share` - 1 others of its shape (the same
+ * sub-graph of other nano-batches on streams of their own; the scheduler's stream assignment at
+ * examples/ae/scheduler/hf/nanoflow.py:122-146 decides that): the launches fill the compute units
+ * together, so K is split less or not at all and the tile shape is chosen for the rounds they take
+ * together.  1 <= share <= 16; share = 1 is dfhip_gemm_bf16_plan. */
+int dfhip_gemm_bf16_plan_shared(int M, int N, int K, int share, int* variant, int* split_k);
 
 /* Split-K flavour of the fast path for shapes with few output tiles (the down
  * projection: [2048,14336] x [4096,14336]^T has 128 tiles of 256x256 for 256
@@ -159,6 +165,12 @@ int dfhip_gemm_bf16_nt_add(const void* A, int64_t lda, const void* W, int64_t ld
 int dfhip_gemm_bf16_gate_up_silu(const void* A, int64_t lda, const void* W_gate, const void* W_up,
                                  int64_t ldw, void* Out, int64_t ldo, int M, int I, int K,
                                  dfhip_stream_t stream);
+/* The same for a launch that runs side by side with `share` - 1 others of its shape (see
+ * dfhip_gemm_bf16_plan_shared): same result bits, the tile shape is chosen for the rounds the launches
+ * take together. */
+int dfhip_gemm_bf16_gate_up_silu_shared(const void* A, int64_t lda, const void* W_gate, const void* W_up,
+                                        int64_t ldw, void* Out, int64_t ldo, int M, int I, int K,
+                                        int share, dfhip_stream_t stream);
 
 /* fp32 in / fp32 accumulate / fp32 out (the CPU-sized fp32 configuration).
  * Requires K % 4 == 0, 16-byte aligned pointers, lda/ldw % 4 == 0. */

@@ -129,12 +129,14 @@ def test_config2_headline_mode_full_size():
         assert torch.equal(again, unfused)
 
 
-def test_config2_down_projections_side_by_side_without_k_split():
-    """``split_k=False`` with one stream per nano-batch: each down projection of a 2048-token nano-batch runs one
-    workgroup per 256 x 256 tile (128 of them) instead of two that split K, and the two nano-batches' projections
-    fill the compute units side by side.  Sampled rows against the oracle; the two-stream issue, the one-stream
-    issue and every replay of the whole-schedule graph have the same bits; within a rounding of the split form."""
-    knobs = dict(fuse_silu_epilogue=True, whole_graph=True, streams="by_nano_batch", split_k=False)
+def test_config2_kernels_planned_for_two_nano_batches_side_by_side():
+    """``side_by_side=2`` with one stream per nano-batch: the same sub-graph of the two nano-batches runs at the same
+    time, and the kernels are planned for the pair.  Each down projection of a 2048-token nano-batch runs one
+    workgroup per 256 x 256 tile (128 of them) instead of two that split K; the gate/up/SiLU launches take the
+    256 x (128 + 128) tile, whose 2 x 896 tiles are exactly 7 rounds of the 256 compute units.  Sampled rows against
+    the oracle; the two-stream issue, the one-stream issue and every replay of the whole-schedule graph have the
+    same bits; within a rounding of the form planned for lone launches (K of the down projection split)."""
+    knobs = dict(fuse_silu_epilogue=True, whole_graph=True, streams="by_nano_batch", side_by_side=2)
     manager, compiled, xg, (x, wg, wu, wd) = build(4096, 4096, 14336, torch.bfloat16, prenorm=True, **knobs)
     eager, split = run(manager, compiled, xg, 4096)
     eager = eager.clone()
@@ -145,13 +147,13 @@ def test_config2_down_projections_side_by_side_without_k_split():
         replay, _ = run(manager, compiled, xg, 4096, use_cudagraph=True)
         assert torch.equal(replay, eager)
     serial_manager, serial, xs, _ = build(4096, 4096, 14336, torch.bfloat16, prenorm=True, serialize=True,
-                                          fuse_silu_epilogue=True, split_k=False)
+                                          fuse_silu_epilogue=True, side_by_side=2)
     one_stream, _ = run(serial_manager, serial, xs, 4096)
     assert torch.equal(one_stream, eager)
-    split_manager, with_split, xk, _ = build(4096, 4096, 14336, torch.bfloat16, prenorm=True, fuse_silu_epilogue=True)
-    split_form, _ = run(split_manager, with_split, xk, 4096)
-    assert not torch.equal(split_form, eager)            # other order of the fp32 additions ...
-    assert rel_err(split_form.float(), eager.float()) < 2 ** -7   # ... and nothing else
+    lone_manager, lone, xk, _ = build(4096, 4096, 14336, torch.bfloat16, prenorm=True, fuse_silu_epilogue=True)
+    lone_form, _ = run(lone_manager, lone, xk, 4096)
+    assert not torch.equal(lone_form, eager)            # other order of the fp32 additions in the down projection ...
+    assert rel_err(lone_form.float(), eager.float()) < 2 ** -7   # ... and nothing else
 
 
 def test_nano_batch_outputs_land_in_one_buffer(monkeypatch):

@@ -192,23 +192,46 @@ def test_stacked_weight_cache_keys_and_lifetime():
     assert len(cache) == 0
 
 
-def test_split_k_option_covers_the_ring_kernel_only():
-    """``launch_options(split_k=False)`` (knob ``split_k``) keeps the 256 x 256 ring kernel (variant 0) from
-    splitting K for the launches issued inside the block; the weight-streaming kernel (variant 6) always splits;
-    the previous setting comes back afterwards, also after an exception."""
-    from dynaflow_amd import ops
+def test_side_by_side_option_and_the_plan_for_shared_launches():
+    """``launch_options(side_by_side=n)`` (knob ``side_by_side``) holds for the launches issued inside the block
+    and comes back afterwards, also after an exception.  The plan for launches that share the GPU (host logic of
+    the library, no GPU needed): the down projection of a 2048-token nano-batch of the 8B shape - 128 tiles of
+    256 x 256 - splits K in two alone and not at all beside a second one; the gate projection keeps its 224-wide
+    tiles either way; decode-sized activations keep the weight-streaming kernel and its split."""
+    import ctypes
+    from dynaflow_amd import _cabi, ops
 
-    assert ops._split_k_on(0) and ops._split_k_on(6)
-    with ops.launch_options(split_k=False):
-        assert not ops._split_k_on(0)
-        assert ops._split_k_on(6)
-        with ops.launch_options(split_k=True):
-            assert ops._split_k_on(0)
-        assert not ops._split_k_on(0)
-    assert ops._split_k_on(0)
+    assert ops._side_by_side() == 1
+    with ops.launch_options(side_by_side=2):
+        assert ops._side_by_side() == 2
+        with ops.launch_options(side_by_side=1):
+            assert ops._side_by_side() == 1
+        assert ops._side_by_side() == 2
     try:
-        with ops.launch_options(split_k=False):
+        with ops.launch_options(side_by_side=4):
             raise RuntimeError("inside")
     except RuntimeError:
         pass
-    assert ops._split_k_on(0)
+    assert ops._side_by_side() == 1
+
+    lib = _cabi.load()
+
+    def plan(M, N, K, share):
+        v, k = ctypes.c_int(), ctypes.c_int()
+        assert lib.dfhip_gemm_bf16_plan_shared(M, N, K, share, ctypes.byref(v), ctypes.byref(k)) == 0
+        return v.value, k.value
+
+    def plan_alone(M, N, K):
+        v, k = ctypes.c_int(), ctypes.c_int()
+        assert lib.dfhip_gemm_bf16_plan(M, N, K, ctypes.byref(v), ctypes.byref(k)) == 0
+        return v.value, k.value
+
+    for shape in ((2048, 4096, 14336), (2048, 14336, 4096), (128, 4096, 4096), (8192, 4096, 4096), (300, 264, 512)):
+        assert plan(*shape, 1) == plan_alone(*shape)
+    assert plan(2048, 4096, 14336, 1) == (0, 2)
+    assert plan(2048, 4096, 14336, 2) == (0, 1)
+    assert plan(1024, 4096, 14336, 2) == (0, 2)          # 64 tiles, twice: still two parts each
+    assert plan(2048, 14336, 4096, 1) == plan(2048, 14336, 4096, 2) == (5, 1)
+    assert plan(128, 4096, 4096, 1) == plan(128, 4096, 4096, 2) and plan(128, 4096, 4096, 2)[0] == 6
+    v, k = ctypes.c_int(), ctypes.c_int()
+    assert lib.dfhip_gemm_bf16_plan_shared(2048, 4096, 14336, 0, ctypes.byref(v), ctypes.byref(k)) == -7
