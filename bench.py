@@ -204,31 +204,34 @@ _PAIR_STREAMS: list = []
 
 
 def time_pair(torch, fn, iters, warmup=20):
-    """Average duration (ms) of two launches that run side by side: ``fn(0)`` on one stream and ``fn(1)`` on another,
-    forked from and joined to the timing stream by events; HIP events on that stream around the loop."""
+    """Average duration (ms) of two launches that run side by side: a loop of ``fn(0)`` on one stream beside a loop of
+    ``fn(1)`` on another (the host issues them alternately, each stream runs its launches back to back); the two
+    streams fork from the timing stream once before the loops and join it once after them, HIP events on that
+    stream around the whole."""
     if not _PAIR_STREAMS:       # made once: streams are dealt to a few hardware queues, and two streams that land
         _PAIR_STREAMS.extend([torch.cuda.Stream(), torch.cuda.Stream()])   # on one queue would run one after the other
     side = _PAIR_STREAMS
     origin = torch.cuda.current_stream()
 
-    def pair():
+    def loops(count):
         fork = torch.cuda.Event()
         fork.record(origin)
-        for i, stream in enumerate(side):
+        for stream in side:
             stream.wait_event(fork)
-            with torch.cuda.stream(stream):
-                fn(i)
+        for _ in range(count):
+            for i, stream in enumerate(side):
+                with torch.cuda.stream(stream):
+                    fn(i)
+        for stream in side:
             join = torch.cuda.Event()
             join.record(stream)
             origin.wait_event(join)
 
-    for _ in range(warmup):
-        pair()
+    loops(warmup)
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
     start.record()
-    for _ in range(iters):
-        pair()
+    loops(iters)
     stop.record()
     stop.synchronize()
     return start.elapsed_time(stop) / iters
@@ -845,8 +848,7 @@ def main() -> int:
                          "frac_of_hbm_peak": silu_bytes / (ms_silu * 1e-3) / 1e9 / HBM_PEAK_GBS},
             "gate_up_silu_gemm": {"ms": ms_gus, "tflops": 2 * gemm_flops / (ms_gus * 1e-3) / 1e12},
             "rocblas_same_gemm_for_scale": {"ms": ms_blas, "tflops": gemm_flops / (ms_blas * 1e-3) / 1e12},
-            # two launches side by side on two streams, kernels planned for the pair; the time includes the fork
-            # from and the join to the timing stream
+            # two loops of launches side by side on two streams, kernels planned for the pair; ms per pair
             "gate_up_silu_gemm_pair": {"ms": ms_gus_pair, "tflops": 4 * gemm_flops / (ms_gus_pair * 1e-3) / 1e12},
             "down_gemm_pair": {"ms": ms_down_pair, "tflops": 2 * gemm_flops / (ms_down_pair * 1e-3) / 1e12},
         },
@@ -856,8 +858,8 @@ def main() -> int:
         result["roofline"] = {
             "kernel": "gemm_bf16_ring_kernel<true> (gate and up projection of one nano-batch with the SiLU*mul epilogue, "
                       "256 x (128 + 128) tile: [2048,4096] x 2 x [14336,4096]^T -> act[2048,14336]); the two "
-                      "nano-batches' launches run side by side on two streams and are timed as a pair, fork and join "
-                      "of the streams included",
+                      "nano-batches' launches run side by side on two streams and are timed as pairs (two loops of "
+                      "launches, one per stream)",
             "bound": "mfma",
             "achieved": 4 * gemm_flops / (ms_gus_pair * 1e-3) / 1e12,
             "peak": BF16_MFMA_PEAK_TFLOPS,
