@@ -541,6 +541,16 @@ def test_planned_gemm_on_seeded_random_shapes(ops, M, N, K):
         fused = ops.gate_up_silu(a, wg, wu)
         separate = ops.silu_mul(ops.linear_variant(a, wg, -2), ops.linear_variant(a, wu, -2), True)
         assert torch.equal(fused, separate)
+    # the same operators planned for launches that share the GPU with one or three others of their shape: another
+    # kernel or split for some shapes, the same product
+    for share in (2, 4):
+        with ops.launch_options(side_by_side=share):
+            y_shared = ops.linear(a, w)
+            err = ((y_shared.float() - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+            assert err <= 2.0 ** -7, (M, N, K, share, err)
+            assert torch.equal(ops.linear_add(a, w, r), r + y_shared)
+            if inter >= 8:
+                assert torch.equal(ops.gate_up_silu(a, wg, wu), separate)
 
 
 @pytest.mark.gpu
