@@ -714,6 +714,14 @@ def main() -> int:
     ms_graph, y_graph = time_steps(torch, m_ovl, c_ovl, x, args.steps, args.warmup, use_graph=True)
     identical = bool(torch.equal(y_serial, y_eager) and torch.equal(y_eager, y_graph))
     y_graph = y_graph.clone()
+    # the same separate kernels with one stream per nano-batch and the kernels planned for the pair (see the fused
+    # modes below): the two nano-batches' launches of each kind run side by side
+    m_op, c_op = build_path(torch, x, weights, whole_graph=True, streams="by_nano_batch", side_by_side=2)
+    ms_graph_pair, y_graph_pair = time_steps(torch, m_op, c_op, x, args.steps, args.warmup, use_graph=True)
+    y_graph_pair = y_graph_pair.clone()
+    m_ops, c_ops = build_path(torch, x, weights, serialize=True, side_by_side=2)
+    _, y_serial_pair = time_steps(torch, m_ops, c_ops, x, 2, 1, use_graph=False)
+    pair_identical = bool(torch.equal(y_serial_pair, y_graph_pair))
 
     # ---- the same layer with the SiLU*mul as the epilogue of one gate/up GEMM
     m_fs, c_fs = build_path(torch, x, weights, serialize=True, whole_graph=True, fuse_silu_epilogue=True)
@@ -810,6 +818,9 @@ def main() -> int:
             "serialized_graph_ms": ms_serial_graph,
             "overlapped_eager_ms": ms_eager,
             "overlapped_graph_ms": ms_graph,
+            "overlapped_graph_stream_per_nano_batch_planned_for_the_pair_ms": ms_graph_pair,
+            "speedup_best_vs_serialized_graph": ms_serial_graph / min(ms_graph, ms_graph_pair),
+            "planned_for_the_pair_bit_identical_to_its_serialized_issue": pair_identical,
             "speedup_eager_vs_serialized": ms_serial / ms_eager,
             "speedup_graph_vs_serialized": ms_serial / ms_graph,
             "speedup_graph_vs_serialized_gpu_side": ms_serial_gpu / ms_graph,
