@@ -254,6 +254,15 @@ size_t counter_area(size_t tiles) {
   return need > 4096 ? need : 4096;
 }
 
+// Which output the W row at position `pos` of a run of paired MFMA blocks belongs to.  MFMA block j = pos / 16
+// hands lane quad q = (pos % 16) / 4 the four outputs r = pos % 4; blocks are paired (0,1), (2,3), ... over 32
+// outputs each, and quad q owns outputs 8q .. 8q+3 of a pair through the even block and 8q+4 .. 8q+7 through the
+// odd one: eight consecutive outputs per lane and pair, one 16-byte store, four lanes a 64-byte run.
+DFHIP_DEVICE int fused_pair_output_of(int pos) {
+  const int j = pos >> 4, n = pos & 15;
+  return 32 * (j >> 1) + 8 * (n >> 2) + 4 * (j & 1) + (n & 3);
+}
+
 // FUSED = false: C[M,N] = A W^T.
 // FUSED = true : C[M,N] = silu(A W^T) * (A W2^T) with W = gate weight, W2 = up weight, N = the
 //   intermediate size.  A tile is 256 rows x 128 columns; its "W half" holds 128 gate rows and 128 up
@@ -301,7 +310,9 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     int ar = m0 + row; ar = ar < M ? ar : M - 1;
     a_off[t] = (uint32_t)((int64_t)(ar - m0) * lda * 2 + chunk * 16);
-    int wr = FUSED ? n0 + (row >> 7) * 64 + (row & 63) : n0 + row;
+    // FUSED: the 64 outputs of a wave column are dealt to its four gate (and four up) MFMA blocks in pairs, so that
+    // a lane ends with 8 consecutive outputs per pair (fused_pair_output_of)
+    int wr = FUSED ? n0 + (row >> 7) * 64 + fused_pair_output_of(row & 63) : n0 + row;
     wr = wr < N ? wr : N - 1;
     w_off[t] = (uint32_t)((int64_t)(wr - n0) * ldw * 2 + chunk * 16);
   }
@@ -450,35 +461,30 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   }
 
   if (FUSED) {
-    // silu(gate) * up in registers, then park 128 rows x 64 columns per wave (144-byte rows)
-    constexpr int FROW_BYTES = 144;
-    uint8_t* park = smem + wave * (128 * FROW_BYTES);
+    // silu(gate) * up in registers (blocks j and j + 4 hold the two projections of the same outputs) and stores
+    // straight from them: 8 consecutive outputs of one row per lane and pair of blocks
+    auto product = [&](int i, int j) {
+      u32x2 packed;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float p[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          // the roundings of the two-kernel path: bf16 projections, bf16 silu, bf16 product
-          const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j][e]));
-          const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][j + 4][e]));
-          p[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
-        }
-        u32x2 v;
-        v[0] = pack2_bf16(p[0], p[1]);
-        v[1] = pack2_bf16(p[2], p[3]);
-        *reinterpret_cast<u32x2*>(park + (i * 16 + frow) * FROW_BYTES + (j * 16 + fquad * 4) * 2) = v;
+      for (int h = 0; h < 2; ++h) {   // two outputs at a time: every rounding is one packed conversion
+        const uint32_t g2 = pack2_bf16(acc[i][j][2 * h], acc[i][j][2 * h + 1]);
+        const uint32_t u2 = pack2_bf16(acc[i][j + 4][2 * h], acc[i][j + 4][2 * h + 1]);
+        const uint32_t s2 = pack2_bf16(silu_fast(bf16_lo_to_f32(g2)), silu_fast(bf16_hi_to_f32(g2)));
+        packed[h] = pack2_bf16(bf16_lo_to_f32(s2) * bf16_lo_to_f32(u2), bf16_hi_to_f32(s2) * bf16_hi_to_f32(u2));
       }
-    DFHIP_PIN;
-    const int m_base = m0 + wave_m * 128, n_base = n0 + wave_n * 64;
-#pragma unroll 4
-    for (int p = 0; p < 16; ++p) {
-      const int id = p * 64 + lane;
-      const int row = id >> 3, c = id & 7;
-      const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * FROW_BYTES + c * 16);
-      const int m = m_base + row, n = n_base + c * 8;
-      if (m < M && n < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n));
+      return packed;
+    };
+    const int m_first = m0 + wave_m * 128 + frow, n_first = n0 + wave_n * 64 + fquad * 8;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int m = m_first + i * 16;
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        const u32x2 even = product(i, 2 * pr), odd = product(i, 2 * pr + 1);
+        const u32x4 v = {even[0], even[1], odd[0], odd[1]};
+        const int n = n_first + pr * 32;   // N % 8 == 0: a run is entirely inside or outside
+        if (m < M && n < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n));
+      }
     }
     return;
   }
@@ -556,12 +562,8 @@ constexpr int TBN = 224;
 // outputs r = pos % 4.  Blocks are paired: (0,1), (2,3), (4,5) cover 32 outputs each, and quad q owns outputs
 // 8q .. 8q+3 of a pair through the even block and 8q+4 .. 8q+7 through the odd one - eight consecutive
 // outputs, one 16-byte store, four lanes a 64-byte run (the size of a write request; with four outputs per lane
-// a tile went out as 32-byte requests, twice as many, and they held up the loads queued behind them).  The
-// seventh block keeps the plain order.
-DFHIP_DEVICE int fused224_output_of(int pos) {
-  const int j = pos >> 4, n = pos & 15;
-  return j < 6 ? 32 * (j >> 1) + 8 * (n >> 2) + 4 * (j & 1) + (n & 3) : pos;
-}
+// a tile went out as twice as many 32-byte requests).  The seventh block keeps the plain order.
+DFHIP_DEVICE int fused224_output_of(int pos) { return pos < 96 ? fused_pair_output_of(pos) : pos; }
 
 template <bool FUSED, int TN>
 __global__ void __launch_bounds__(RTHREADS)
