@@ -863,6 +863,23 @@ def main() -> int:
             "gate_up_silu_gemm_pair": {"ms": ms_gus_pair, "tflops": 4 * gemm_flops / (ms_gus_pair * 1e-3) / 1e12},
             "down_gemm_pair": {"ms": ms_down_pair, "tflops": 2 * gemm_flops / (ms_down_pair * 1e-3) / 1e12},
         },
+        # the reference's stand-alone experiment (examples/ae/up-silu-overlap.cu:320-341: GEMM only, SiLU only,
+        # serial = their sum, the fused kernel, speedup = serial / fused, FUSED / GEMM) on one nano-batch of this
+        # layer, from the single-kernel loops above: the GEMM is the gate and the up projection as two launches
+        "gate_up_silu_experiment": {
+            "gemm_only_us": 2e3 * ms_gate,
+            "silu_only_us": 1e3 * ms_silu,
+            "serial_us": 2e3 * ms_gate + 1e3 * ms_silu,
+            "fused_us": 1e3 * ms_gus,
+            "speedup_fused_vs_serial": (2 * ms_gate + ms_silu) / ms_gus,
+            "fused_over_gemm_only": ms_gus / (2 * ms_gate),
+            "fused_us_beside_the_other_nano_batch": 0.5e3 * ms_gus_pair,
+            "speedup_fused_beside_the_other_nano_batch_vs_serial": (2 * ms_gate + ms_silu) / (0.5 * ms_gus_pair),
+        },
+        # the layer the same way: separate GEMM and SiLU*mul launches of both nano-batches one after the other on
+        # one stream (the reference's serial baseline) against the issue mode that `value` comes from
+        "speedup_best_vs_serialized_separate_kernels": ms_serial / best_ms,
+        "speedup_best_vs_serialized_separate_kernels_graph": ms_serial_graph / best_ms,
     }
     # the dominant kernel of the issue mode that `value` comes from
     if fused_wins and best_fused_mode.endswith("kernels_planned_for_the_pair"):
