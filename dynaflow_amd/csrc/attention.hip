@@ -1,7 +1,10 @@
 // Causal grouped-query attention for prefill (bf16, head_dim 128), flash-attention style: scores and
 // probabilities never leave the registers.
 //
-// One workgroup = 256 query rows of one (sequence, query head); 4 waves x 64 rows.  K and V are staged
+// One workgroup = 4 waves x 64 query rows that share one (sequence, kv head): the same 64 rows of 4 query heads
+// of the group (HPW = 4: every wave has the same diagonal block, so no wave waits for another one's masked
+// tiles, and no tile lies wholly above the diagonal), 128 rows of 2 heads, or 256 rows of one head, whichever
+// the group size allows.  K and V are staged
 // in LDS in blocks of 64 positions by LDS-DMA (3 stages in flight).  Both products are computed
 // transposed so that no operand ever needs a transpose:
 //   S^T[pos, qrow] = K Q^T   A = K rows from LDS, B = Q fragments held in registers for the whole kernel
@@ -27,7 +30,7 @@
 namespace {
 
 constexpr int AD = 128;          // head dim
-constexpr int QROWS = 256;       // query rows per workgroup
+constexpr int WAVE_ROWS = 64;    // query rows per wave
 constexpr int KVB = 64;          // positions per staged block
 constexpr int STAGES = 4;
 constexpr int K_BYTES = KVB * AD * 2;            // 16 KiB
@@ -49,11 +52,13 @@ DFHIP_DEVICE int pi(int m) {   // MFMA row -> position inside a 32-position tile
   return (m & 16) | (g2 << 2) | (m & 3);
 }
 
-// workgroup -> (sequence, kv head, query head, query block).  All query heads of a (sequence, kv head)
-// pair run on ONE XCD (its K and V stay in that XCD's L2); inside an XCD's range the heavy query blocks
-// (late rows, many K/V blocks) come first.
+// workgroup -> (sequence, kv head, first query head, query block) for workgroups of HPW heads x QROWS rows.  All
+// query heads of a (sequence, kv head) pair run on ONE XCD (its K and V stay in that XCD's L2); inside an XCD's
+// range the heavy query blocks (late rows, many K/V blocks) come first.
+template <int HPW>
 DFHIP_DEVICE void map_workgroup(int B, int S, int q_heads, int kv_heads, int& b, int& kvh, int& hq, int& qb) {
-  const int group = q_heads / kv_heads;
+  constexpr int QROWS = WAVE_ROWS * 4 / HPW;
+  const int group = q_heads / kv_heads / HPW;    // workgroups per (sequence, kv head, query block)
   const int nqb = (S + QROWS - 1) / QROWS;
   const int sets = B * kv_heads;
   int hg;
@@ -77,7 +82,7 @@ DFHIP_DEVICE void map_workgroup(int B, int S, int q_heads, int kv_heads, int& b,
     b = set / kv_heads;
     kvh = set % kv_heads;
   }
-  hq = kvh * group + hg;
+  hq = (kvh * group + hg) * HPW;
 }
 
 // The fast pass is software-pipelined: with one wave per SIMD nothing else fills the matrix pipe while a
@@ -85,6 +90,7 @@ DFHIP_DEVICE void map_workgroup(int B, int S, int q_heads, int kv_heads, int& b,
 // pinned - the P V MFMAs of tile t, the score MFMAs of tile t+2, and the softmax (VALU) of tile t+1.  Score
 // tiles and probability fragments alternate between two register sets (A: even tiles, B: odd tiles).  K/V
 // blocks live in a ring of 4 stages: block j (V in use), j+1 (K in use), j+2 and j+3 landing.
+template <int HPW>
 __global__ void __launch_bounds__(256)
 causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint16_t* __restrict__ k, int64_t ld_k,
                         const uint16_t* __restrict__ v_blk, uint16_t* __restrict__ out, int64_t ld_o, int B, int S,
@@ -93,11 +99,15 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 31, half = lane >> 5;
+  constexpr int WPH = 4 / HPW;                 // waves per head
+  constexpr int QROWS = WAVE_ROWS * WPH;       // query rows per workgroup
   int b, kvh, hq, qb;
-  map_workgroup(B, S, q_heads, kv_heads, b, kvh, hq, qb);
+  map_workgroup<HPW>(B, S, q_heads, kv_heads, b, kvh, hq, qb);
+  hq += wave / WPH;                            // this wave's query head ...
+  const int wrow = wave % WPH;                 // ... and its 64 rows of the workgroup's query block
   const int q0 = qb * QROWS;
   const int last_block_wg = ((q0 + QROWS < S ? q0 + QROWS : S) + KVB - 1) / KVB - 1;
-  int last_block_wave = q0 / KVB + wave;                        // the wave's diagonal block
+  int last_block_wave = q0 / KVB + wrow;                        // the wave's diagonal block
   if (last_block_wave > last_block_wg) last_block_wave = last_block_wg;   // a wave of rows past S (never stored)
 
   // ---- DMA sources: uniform bases that advance by one block, per-lane offsets fixed for the whole kernel
@@ -137,7 +147,7 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
   bf16x8 qf[2][8];
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb) {
-    int qrow = q0 + wave * 64 + nb * 32 + col;
+    int qrow = q0 + wrow * WAVE_ROWS + nb * 32 + col;
     qrow = qrow < S ? qrow : S - 1;
     const uint16_t* qp = q + ((int64_t)b * S + qrow) * ld_q + (int64_t)hq * AD + 8 * half;
 #pragma unroll
@@ -153,7 +163,7 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[db][nb][r] = 0.0f;
   const int k_read = col * 256;
-  const int my_qrow0 = q0 + wave * 64 + col;
+  const int my_qrow0 = q0 + wrow * WAVE_ROWS + col;
 
   // LDS addresses of the A fragments: V pair p = (t, db) of tile [block, sb], K k-step ks of tile [block, sb]
   auto v_frag = [&](int block, int sb, int p) {
@@ -327,7 +337,7 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
       const float inv = 1.0f / row_sum[nb];
-      const int qrow = q0 + wave * 64 + nb * 32 + col;
+      const int qrow = q0 + wrow * WAVE_ROWS + nb * 32 + col;
       uint16_t* orow = out + ((int64_t)b * S + qrow) * ld_o + (int64_t)hq * AD + 4 * half;
       if (qrow < S) {
 #pragma unroll
@@ -474,7 +484,10 @@ extern "C" int dfhip_causal_attention_bf16(const void* q, int64_t ld_q, const vo
   if (!q || !k || !v_blk || !out) return DFHIP_ERR_NULL_POINTER;
   if (B < 1 || S < KVB || S % KVB != 0 || q_heads < 1 || kv_heads < 1 || q_heads % kv_heads != 0 || head_dim != AD)
     return DFHIP_ERR_BAD_SHAPE;
-  const int64_t groups = (int64_t)B * q_heads * ((S + QROWS - 1) / QROWS);
+  const int group = q_heads / kv_heads;
+  const int hpw = group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;      // query heads per workgroup
+  const int wg_rows = WAVE_ROWS * 4 / hpw;
+  const int64_t groups = (int64_t)B * (q_heads / hpw) * ((S + wg_rows - 1) / wg_rows);
   if (groups >= (int64_t)1 << 31) return DFHIP_ERR_BAD_SHAPE;
   if (ld_q < (int64_t)q_heads * AD || ld_k < (int64_t)kv_heads * AD || ld_o < (int64_t)q_heads * AD ||
       ld_k >= (int64_t)1 << 24)   // a K block's byte offsets are kept in 32 bits
@@ -482,11 +495,18 @@ extern "C" int dfhip_causal_attention_bf16(const void* q, int64_t ld_q, const vo
   if (ld_q % 8 || ld_k % 8 || ld_o % 8 || !dfhip_aligned16(q) || !dfhip_aligned16(k) || !dfhip_aligned16(v_blk) ||
       !dfhip_aligned16(out))
     return DFHIP_ERR_BAD_ALIGNMENT;
-  static std::atomic<uint64_t> lds_opted_in{0};   // per instantiation, one bit per device
-  if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(causal_attention_kernel), ATT_LDS, lds_opted_in)) return rc;
-  hipLaunchKernelGGL(causal_attention_kernel, dim3((unsigned)groups), dim3(256), ATT_LDS,
-                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(q), ld_q,
-                     static_cast<const uint16_t*>(k), ld_k, static_cast<const uint16_t*>(v_blk),
-                     static_cast<uint16_t*>(out), ld_o, B, S, q_heads, kv_heads, scale * 1.4426950408889634f);
-  return dfhip_check_launch();
+  auto launch = [&](auto heads_per_workgroup) {
+    constexpr int HPW = decltype(heads_per_workgroup)::value;
+    static std::atomic<uint64_t> lds_opted_in{0};   // per instantiation, one bit per device
+    if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(causal_attention_kernel<HPW>), ATT_LDS, lds_opted_in))
+      return rc;
+    hipLaunchKernelGGL(causal_attention_kernel<HPW>, dim3((unsigned)groups), dim3(256), ATT_LDS,
+                       static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(q), ld_q,
+                       static_cast<const uint16_t*>(k), ld_k, static_cast<const uint16_t*>(v_blk),
+                       static_cast<uint16_t*>(out), ld_o, B, S, q_heads, kv_heads, scale * 1.4426950408889634f);
+    return dfhip_check_launch();
+  };
+  if (hpw == 4) return launch(std::integral_constant<int, 4>{});
+  if (hpw == 2) return launch(std::integral_constant<int, 2>{});
+  return launch(std::integral_constant<int, 1>{});
 }

@@ -30,7 +30,7 @@ def inputs(B, S, Hq, Hkv, seed):
 
 
 @pytest.mark.parametrize("B,S,Hq,Hkv", [(1, 64, 1, 1), (2, 128, 4, 2), (3, 320, 8, 2), (1, 512, 4, 1), (2, 256, 3, 3),
-                                        (8, 64, 4, 1)])
+                                        (8, 64, 4, 1), (1, 192, 2, 1), (1, 320, 3, 1), (1, 128, 8, 1)])
 def test_causal_attention_against_oracle(ops, B, S, Hq, Hkv):
     q, k, v = inputs(B, S, Hq, Hkv, S + Hq)
     print(f"causal attention B={B} S={S} Hq={Hq} Hkv={Hkv}", flush=True)
