@@ -138,6 +138,17 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
 #pragma unroll
     for (int t = 0; t < 8; ++t) issue_piece(j, t);
   };
+  // The same for the steps of the main loop, without a branch: a piece past the last block re-reads the last
+  // block into the stage that its own block would have taken, which nobody reads any more.  (A branch here cuts
+  // the step into basic blocks, and the compiler then sinks the step's softmax across them to its first use in
+  // the next step: 32 exponentials in one run with no MFMA over them.)
+  auto issue_piece_or_dummy = [&](int j, int t) {
+    const int src = j < last_block_wg ? j : last_block_wg;
+    const int stage = j % STAGES;
+    if (t < 4) dma16_base(stage * STAGE_BYTES + (wave * 4 + t) * 1024, kseq + src * k_block_bytes, k_off[t]);
+    else dma16_base(stage * STAGE_BYTES + K_BYTES + (wave * 4 + t - 4) * 1024, vseq + (int64_t)src * (KVB * AD * 2),
+                    v_off[t - 4]);
+  };
 
   issue_block(0);
   issue_block(1);
@@ -192,21 +203,27 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
       neg_ref[nb] = -fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * scale_log2;
     }
   };
-  // The softmax of one score tile in the fast pass is 16 slices (8 per half of the query rows), small enough
-  // to sit behind one MFMA each: a slice turns two scores into probabilities.  No maximum is taken and no
-  // sum: the row sums come out of the matrix pipe (an all-ones A operand against the probabilities), and
-  // whether a row's scores outgrew its reference shows in that sum at the end.
+  // The softmax of one score tile in the fast pass is 32 slices (16 per half of the query rows), one behind
+  // nearly every MFMA of a step: a slice turns one score into a probability (an even register's waits for its
+  // odd neighbour to be packed with it).  No maximum is taken and no sum: the row sums come out of the matrix
+  // pipe (an all-ones A operand against the probabilities), and whether a row's scores outgrew its reference
+  // shows in that sum at the end.
+  float held = 0.0f;                          // the probability of an even register until its odd neighbour follows
   auto softmax_slice = [&](auto diag, int i, int block, int sb, const f32x16 (&s)[2], bf16x8 (&pf)[2][2]) {
-    const int nb = i >> 3, r = 2 * (i & 7);
-    float x0 = s[nb][r], x1 = s[nb][r + 1];
+    const int nb = i >> 4, r = i & 15;
+    float x = s[nb][r];
     if (decltype(diag)::value) {
       const int pos = block * KVB + sb * 32 + 8 * half + 16 * (r >> 3) + (r & 7);
       const int qrow = my_qrow0 + 32 * nb;
-      if (pos > qrow) x0 = -INFINITY;
-      if (pos + 1 > qrow) x1 = -INFINITY;
+      if (pos > qrow) x = -INFINITY;
     }
-    pf[nb][r >> 3][r & 7] = static_cast<bf16_t>(__builtin_amdgcn_exp2f(fmaf(x0, scale_log2, neg_ref[nb])));
-    pf[nb][r >> 3][(r & 7) + 1] = static_cast<bf16_t>(__builtin_amdgcn_exp2f(fmaf(x1, scale_log2, neg_ref[nb])));
+    const float e = __builtin_amdgcn_exp2f(fmaf(x, scale_log2, neg_ref[nb]));
+    if (r & 1) {
+      pf[nb][r >> 3][(r & 7) - 1] = static_cast<bf16_t>(held);
+      pf[nb][r >> 3][r & 7] = static_cast<bf16_t>(e);
+    } else {
+      held = e;
+    }
   };
 
   // One step: P V of tile [vb, vsb] (probabilities pf_in) with the two row-sum MFMAs of each k-step behind
@@ -241,7 +258,7 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
       // the 8 LDS-DMA instructions of the block that enters the ring in this iteration, spread over the step
       // (4 waves issuing them in one burst keep the address unit, and with it the waves, busy for ~500 cycles)
       if (dma_block >= 0) {
-        if (DO_S ? (pq & 1) && pq < 16 : pq < 8) issue_piece(dma_block, DO_S ? pq >> 1 : pq);
+        if (DO_S ? (pq & 1) && pq < 16 : pq < 8) issue_piece_or_dummy(dma_block, DO_S ? pq >> 1 : pq);
       }
       if (!is_sum) {
         const int n = f + AHEAD;               // the fragment to fetch now
@@ -263,9 +280,9 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
           s_out[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[f], qf[nb][f - 8], s_out[nb], 0, 0, 0);
         }
         if (DO_SM) {
-          const int m = 2 * pq + nb;           // slices [16 m / (2 PAIRS), 16 (m+1) / (2 PAIRS))
+          const int m = 2 * pq + nb;           // slices [32 m / (2 PAIRS), 32 (m+1) / (2 PAIRS))
 #pragma unroll
-          for (int i = 16 * m / (2 * PAIRS); i < 16 * (m + 1) / (2 * PAIRS); ++i)
+          for (int i = 32 * m / (2 * PAIRS); i < 32 * (m + 1) / (2 * PAIRS); ++i)
             softmax_slice(diag, i, mb, msb, s_in, pf_out);
         }
         DFHIP_PIN;
@@ -299,10 +316,10 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
   first_tile_reference(last_block_wave == 0, sA);
   if (last_block_wave == 0) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) softmax_slice(yes{}, i, 0, 0, sA, pfA);
+    for (int i = 0; i < 32; ++i) softmax_slice(yes{}, i, 0, 0, sA, pfA);
   } else {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) softmax_slice(no{}, i, 0, 0, sA, pfA);
+    for (int i = 0; i < 32; ++i) softmax_slice(no{}, i, 0, 0, sA, pfA);
   }
 #pragma unroll
   for (int a = 0; a < AHEAD; ++a) vpre[a] = v_frag(0, 0, a);
@@ -316,21 +333,28 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
     else wait_vmcnt<0>();
     workgroup_barrier();                     // block j+1 is there for every wave; everybody is done with block j-1
   };                                         // ... so block j+3 may enter the ring (first step of the iteration)
+  // While a wave runs steps, every iteration issues exactly 8 pieces (block j+3 or its stand-in), so "at most 8
+  // in flight" always means that block j+1 has landed.
+  auto turn_ring_in_steps = [&]() {
+    wait_vmcnt<8>();
+    workgroup_barrier();
+  };
   int j = 0;
   for (; j + 1 < last_block_wave; ++j) {
-    turn_ring(j);
+    turn_ring_in_steps();
     step(yes{}, yes{}, no{}, j, 0, pfA, j + 1, 0, sA, j, 1, sB, pfB, j, 1, j + 3);
     step(yes{}, yes{}, no{}, j, 1, pfB, j + 1, 1, sB, j + 1, 0, sA, pfA, j + 1, 0, NO_DMA);
   }
   if (j < last_block_wave) {                 // the block before the diagonal one: its second softmax is masked
-    turn_ring(j);
+    turn_ring_in_steps();
     step(yes{}, yes{}, no{}, j, 0, pfA, j + 1, 0, sA, j, 1, sB, pfB, j, 1, j + 3);
     step(yes{}, yes{}, yes{}, j, 1, pfB, j + 1, 1, sB, j + 1, 0, sA, pfA, j + 1, 0, NO_DMA);
     ++j;
   }
-  turn_ring(j);
+  turn_ring_in_steps();
   step(no{}, yes{}, yes{}, j, 0, pfA, 0, 0, sA, j, 1, sB, pfB, j, 1, j + 3);
   step(no{}, no{}, no{}, j, 1, pfB, 0, 0, sA, 0, 0, sB, pfA, j, 1, NO_DMA);
+  wait_vmcnt<0>();                           // the last pieces (stand-ins, possibly) are out of the way of what follows
   // The output goes from the registers straight to memory (a lane holds runs of 4 dims of its query rows), so
   // a wave that is done stores while the others still work; its remaining duty is the ring.
   auto store_rows = [&](const float (&row_sum)[2]) {
