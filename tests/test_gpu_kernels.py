@@ -568,3 +568,28 @@ def test_planned_fp8_gemm_on_assorted_shapes(ops, M, N, K):
     want = (xq.float() * xs) @ (wq.float() * ws[:, None]).t()
     err = ((got.float() - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
     assert err <= 2.0 ** -6, (M, N, K, err)
+
+
+def test_zero_row_inputs_give_empty_outputs(ops):
+    """A nano-batch without tokens (a split index repeated) reaches the operators as a [0, H] tensor: every
+    operator returns the empty tensor of the right shape and launches nothing; the C ABI itself refuses M = 0."""
+    from dynaflow_amd import _cabi
+
+    H, I = 128, 256
+    x = torch.zeros(0, H, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(I, H, dtype=torch.bfloat16, device="cuda")
+    wd = torch.zeros(H, I, dtype=torch.bfloat16, device="cuda")
+    act = ops.gate_up_silu(x, w, w)
+    assert act.shape == (0, I) and act.dtype == torch.bfloat16
+    assert ops.linear(x, w).shape == (0, I)
+    assert ops.silu_mul(ops.linear(x, w), ops.linear(x, w), True).shape == (0, I)
+    assert ops.linear(act, wd).shape == (0, H)
+    assert ops.linear_add(act, wd, x).shape == (0, H)
+    assert ops.rms_norm(x, torch.ones(H, dtype=torch.bfloat16, device="cuda"), 1e-5).shape == (0, H)
+    both = ops.linear_multi(x, [w, w])
+    assert [tuple(t.shape) for t in both] == [(0, I), (0, I)]
+    x32 = torch.zeros(0, H, device="cuda")
+    assert ops.linear(x32, w.float()).shape == (0, I)
+    lib = _cabi.load()
+    rc = lib.dfhip_gemm_bf16_nt(w.data_ptr(), H, w.data_ptr(), H, w.data_ptr(), I, 0, I, H, 0)
+    assert rc == -2          # DFHIP_ERR_BAD_SHAPE
