@@ -46,6 +46,23 @@ DFHIP_DEVICE float max3(float a, float b, float c) {
   return r;
 }
 
+// The score products of the fast pass, written out with their register classes: the result tile in VECTOR
+// registers, where the softmax reads it with ordinary instructions, and the Q fragment - which is only ever an MFMA
+// operand - in ACCUMULATION registers.  Left to the compiler the score tiles sit in accumulation registers and
+// every score costs a v_accvgpr_read_b32, which beside running MFMAs takes about three times as long as an
+// ordinary vector instruction (take-it-out timing).  The compiler does not know that these are MFMAs: a result is
+// first read two or more MFMAs (64 cycles) after the last product into it, which covers the 11 wait states of an
+// 8-pass MFMA; the accumulating form reads exactly the registers it writes, the one dependent sequence that the
+// matrix pipe forwards by itself.
+DFHIP_DEVICE f32x16 mfma_scores_first(bf16x8 k_rows, bf16x8 q_frag) {
+  f32x16 d;
+  asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(k_rows), "a"(q_frag));
+  return d;
+}
+DFHIP_DEVICE void mfma_scores_next(f32x16& d, bf16x8 k_rows, bf16x8 q_frag) {
+  asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(k_rows), "a"(q_frag));
+}
+
 DFHIP_DEVICE int pi(int m) {   // MFMA row -> position inside a 32-position tile
   const int g = (m >> 2) & 3;
   const int g2 = ((g & 1) << 1) | (g >> 1);      // 0,1,2,3 -> 0,2,1,3
@@ -274,10 +291,9 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
           const int t = f >> 2, db = f & 3;
           o[db][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[f], pf_in[nb][t], o[db][nb], 0, 0, 0);
         } else if (f == 8) {
-          const f32x16 zero = {};
-          s_out[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[f], qf[nb][0], zero, 0, 0, 0);
+          s_out[nb] = mfma_scores_first(fr[f], qf[nb][0]);
         } else {
-          s_out[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[f], qf[nb][f - 8], s_out[nb], 0, 0, 0);
+          mfma_scores_next(s_out[nb], fr[f], qf[nb][f - 8]);
         }
         if (DO_SM) {
           const int m = 2 * pq + nb;           // slices [32 m / (2 PAIRS), 32 (m+1) / (2 PAIRS))
@@ -299,6 +315,11 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
   bf16x8 pfA[2][2], pfB[2][2];
   wait_vmcnt<0>();                           // Q and the first blocks have landed
   workgroup_barrier();
+  // from here on the Q fragments live in accumulation registers (see mfma_scores_first)
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+a"(qf[nb][ks]));
   // prologue (not overlapped): scores of tiles 0 and 1, softmax of tile 0
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
@@ -308,8 +329,8 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
       const bf16x8 kf = k_frag(0, t, ks);
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb) {
-        const f32x16 zero = {};
-        sd[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[nb][ks], ks == 0 ? zero : sd[nb], 0, 0, 0);
+        if (ks == 0) sd[nb] = mfma_scores_first(kf, qf[nb][0]);
+        else mfma_scores_next(sd[nb], kf, qf[nb][ks]);
       }
     }
   }
