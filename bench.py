@@ -448,7 +448,10 @@ def decoder_config(torch, steps, warmup):
     T = batch * S
     results = {}
     for name, knobs in (("serialized", {"serialize": True}), ("overlapped", {"whole_graph": True}),
-                        ("overlapped_fused_silu", {"whole_graph": True, "fuse_silu_epilogue": True})):
+                        ("overlapped_fused_silu", {"whole_graph": True, "fuse_silu_epilogue": True}),
+                        # every nano-batch on a stream of its own instead of one stream per kind of sub-graph
+                        ("stream_per_nano_batch_fused_silu", {"whole_graph": True, "fuse_silu_epilogue": True,
+                                                              "streams": "by_nano_batch"})):
         extra = {"min_nano_split_tokens": 64, "dump_graph": False, **EXTRA_KNOBS}
         extra.update(knobs)
         cfg = DynaFlowConfig("dynaflow_amd.schedulers:DecoderOverlapScheduler", 2, InductorConfig(enabled=True),
@@ -473,8 +476,10 @@ def decoder_config(torch, steps, warmup):
                 torch.cuda.synchronize()
                 results[f"{name}_{mode}_ms"] = (time.perf_counter() - t0) * 1e3 / steps
     flops = 2.0 * T * H * 6144 + 2.0 * T * H * H + 2.0 * batch * 32 * S * S * 128 + 6.0 * T * H * I
-    best = min(results["overlapped_graph_ms"], results["overlapped_eager_ms"],
-               results["overlapped_fused_silu_graph_ms"])
+    candidates = ("overlapped_graph_ms", "overlapped_eager_ms", "overlapped_fused_silu_graph_ms",
+                  "stream_per_nano_batch_fused_silu_graph_ms")
+    best_mode = min(candidates, key=lambda m: results[m])
+    best = results[best_mode]
     # the dominant kernel, alone: gate + up + SiLU*mul of one nano-batch (8192 tokens) in one launch
     from dynaflow_amd import ops
     mb = T // 2
@@ -492,7 +497,8 @@ def decoder_config(torch, steps, warmup):
         "config": {"workload": "Llama-3-8B-shaped decoder layer, prefill 8 x 2048 tokens, 2 nano-batches of 4 "
                                "sequences, attention sub-graph of one beside the MLP sub-graph of the other; "
                                "projections, RoPE, causal attention, norms and MLP on the hand-written HIP "
-                               "operators (embedding gather, residual adds and the final concatenation on aten)"},
+                               "operators (embedding gather, residual adds and the final concatenation on aten)",
+                   "issue_mode": best_mode[:-3]},
         "timings": results,
         "layer": {"algorithmic_tflop": flops / 1e12, "tflops": flops / (best * 1e-3) / 1e12,
                   "frac_of_bf16_mfma_peak": flops / (best * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS},
