@@ -77,3 +77,16 @@ def test_missing_library_is_loud(monkeypatch):
     monkeypatch.setattr(_cabi, "LIB_PATH", "/nonexistent/libdynaflow_hip.so")
     with pytest.raises(_cabi.KernelLibraryMissing):
         _cabi.load()
+
+
+def test_header_is_plain_c_and_cpp():
+    """The boundary is a C ABI: the header must go through a C99 compiler (no C++ in the signatures) and through a
+    C++ compiler alike."""
+    import shutil
+    import subprocess
+
+    gcc, gpp = shutil.which("gcc"), shutil.which("g++")
+    if not gcc or not gpp:
+        pytest.skip("no host compiler")
+    subprocess.run([gcc, "-fsyntax-only", "-x", "c", "-std=c99", "-Wall", "-Werror", "-pedantic", HEADER], check=True)
+    subprocess.run([gpp, "-fsyntax-only", "-x", "c++", "-std=c++11", "-Wall", "-Werror", HEADER], check=True)
