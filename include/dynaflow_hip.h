@@ -56,7 +56,9 @@ typedef struct dfhip_device_info {
   char arch_name[64];      /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
 } dfhip_device_info;
 
-/* Library ABI version (major*1000 + minor). */
+/* Library ABI version (major*1000 + minor).  This and the next two have no counterpart in the
+ * reference (its sub-graphs call PyTorch, dynaflow/runtime/engine.py:381, which reports its own
+ * errors): housekeeping for whoever binds the library. */
 int dfhip_version(void);
 /* The architecture the device code was compiled for ("gfx950"). */
 const char* dfhip_arch(void);
@@ -79,7 +81,9 @@ int dfhip_device_info_get(int device, dfhip_device_info* out);
 int dfhip_gemm_bf16_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                        int64_t ldc, int M, int N, int K, dfhip_stream_t stream);
 
-/* Same contraction with an explicit kernel variant, for tuning and tests.
+/* Same contraction (the `linear` node, dynaflow/runtime/engine.py:381) with an explicit kernel
+ * variant, for tuning and tests; the choice itself has no counterpart in the reference, where
+ * PyTorch picks its GEMM kernel out of sight.
  * variant: 0 = 256x256 tile, LDS-DMA ring (the fast path);
  *          5 = 256x224 tile, LDS-DMA ring (chosen when N = 7 * 2^k makes 224-wide
  *              tiles fill the rounds of 256 workgroups better, e.g. N = 14336);
@@ -95,7 +99,8 @@ int dfhip_gemm_bf16_nt_variant(const void* A, int64_t lda, const void* W, int64_
                                int64_t ldc, int M, int N, int K, int variant,
                                dfhip_stream_t stream);
 
-/* The kernel choice dfhip_gemm_bf16_nt makes for a shape (variant as above) and
+/* The kernel choice dfhip_gemm_bf16_nt makes for a shape (variant as above; no counterpart in the
+ * reference, see there) and
  * the split_k a caller with a workspace should pass to dfhip_gemm_bf16_nt_splitk
  * (1 = no split). */
 int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* split_k);
@@ -106,8 +111,9 @@ int dfhip_gemm_bf16_plan(int M, int N, int K, int* variant, int* split_k);
  * together.  1 <= share <= 16; share = 1 is dfhip_gemm_bf16_plan. */
 int dfhip_gemm_bf16_plan_shared(int M, int N, int K, int share, int* variant, int* split_k);
 
-/* Split-K flavour of the fast path for shapes with few output tiles (the down
- * projection: [2048,14336] x [4096,14336]^T has 128 tiles of 256x256 for 256
+/* Split-K flavour of the fast path for shapes with few output tiles (the same `linear` node,
+ * dynaflow/runtime/engine.py:381; the down projection of the host model's MLP, whose gate and up
+ * projections examples/ae/scheduler/hf/nanoflow.py:30 names: [2048,14336] x [4096,14336]^T has 128 tiles of 256x256 for 256
  * compute units).  Each tile is computed by `split_k` workgroups over disjoint
  * K ranges.  With the 256x256 ring kernel parts 0 .. split_k-2 leave their fp32
  * block in `workspace` and count themselves in; the last part - the one with the
@@ -145,7 +151,8 @@ int dfhip_gemm_bf16_nt_splitk_static(const void* A, int64_t lda, const void* W, 
                                      dfhip_stream_t stream);
 
 /* C[M,N] = bf16( bf16(A W^T) + R ): the contraction with the residual addition
- * that follows it in a decoder layer (FX nodes linear, add) as the epilogue of the
+ * that follows it in a decoder layer (FX nodes linear, add of the host model traced by
+ * examples/ae/scripts/bench_hf_transformers.py:206-210, run at dynaflow/runtime/engine.py:381) as the epilogue of the
  * kernel dfhip_gemm_bf16_plan picks.  R is [M,N] with the leading dimension of C;
  * the roundings are those of the separate linear and add kernels, so the bits are
  * the same.  split_k and workspace as in dfhip_gemm_bf16_nt_splitk (split_k = 1:
@@ -156,7 +163,9 @@ int dfhip_gemm_bf16_nt_add(const void* A, int64_t lda, const void* W, int64_t ld
 
 /* Gate and up projection with the SiLU*mul as the GEMM's epilogue:
  *   Out[M,I] = bf16( silu(A W_gate^T) * (A W_up^T) )
- * - the FX nodes linear, linear, silu, mul of the MLP in one launch.  Both
+ * - the FX nodes linear, linear, silu, mul of the MLP (gate_proj and up_proj of
+ * examples/ae/scheduler/hf/nanoflow.py:30, SiLU*mul as in examples/ae/up-silu-overlap.cu:75-90) in one
+ * launch, the job of the reference's fused kernel (examples/ae/up-silu-overlap.cu:119-181).  Both
  * weights [I,K] with the same leading dimension ldw.  The epilogue applies
  * the roundings of the separate kernels (projections to bf16, silu to bf16,
  * product to bf16), so the result has the same bits as dfhip_gemm_bf16_nt
@@ -166,18 +175,22 @@ int dfhip_gemm_bf16_gate_up_silu(const void* A, int64_t lda, const void* W_gate,
                                  int64_t ldw, void* Out, int64_t ldo, int M, int I, int K,
                                  dfhip_stream_t stream);
 /* The same for a launch that runs side by side with `share` - 1 others of its shape (see
- * dfhip_gemm_bf16_plan_shared): same result bits, the tile shape is chosen for the rounds the launches
+ * dfhip_gemm_bf16_plan_shared; streams as assigned at examples/ae/scheduler/hf/nanoflow.py:122-146):
+ * same result bits, the tile shape is chosen for the rounds the launches
  * take together. */
 int dfhip_gemm_bf16_gate_up_silu_shared(const void* A, int64_t lda, const void* W_gate, const void* W_up,
                                         int64_t ldw, void* Out, int64_t ldo, int M, int I, int K,
                                         int share, dfhip_stream_t stream);
 
-/* fp32 in / fp32 accumulate / fp32 out (the CPU-sized fp32 configuration).
+/* fp32 in / fp32 accumulate / fp32 out (the `linear` node, dynaflow/runtime/engine.py:381, of the
+ * CPU-sized fp32 configuration).
  * Requires K % 4 == 0, 16-byte aligned pointers, lda/ldw % 4 == 0. */
 int dfhip_gemm_f32_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                       int64_t ldc, int M, int N, int K, dfhip_stream_t stream);
 
-/* fp8 e4m3fn inputs, fp32 accumulate, bf16 output:
+/* fp8 e4m3fn inputs, fp32 accumulate, bf16 output (the `linear` node, dynaflow/runtime/engine.py:381,
+ * of a host model whose weights are quantised per output channel and whose activations are
+ * quantised per tensor):
  *   C[m,n] = bf16( a_scale[0] * w_scale[n] * sum_k A[m,k] * W[n,k] )
  * a_scale: device pointer to ONE float (per-tensor dynamic scale),
  * w_scale: device pointer to N floats (per-output-channel scale).
@@ -185,7 +198,8 @@ int dfhip_gemm_f32_nt(const void* A, int64_t lda, const void* W, int64_t ldw, vo
 int dfhip_gemm_fp8_nt(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                       int64_t ldc, const float* a_scale, const float* w_scale, int M, int N,
                       int K, dfhip_stream_t stream);
-/* The same with an explicit kernel, for tuning and tests: 0 = 256x256 LDS-DMA ring,
+/* The same with an explicit kernel, for tuning and tests (the choice has no counterpart in the
+ * reference): 0 = 256x256 LDS-DMA ring,
  * 1 = register-staged 128x128, 2 = 256x224 LDS-DMA ring (N = 7 * 2^k), negative =
  * the choice dfhip_gemm_fp8_nt makes. */
 int dfhip_gemm_fp8_nt_variant(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
@@ -217,7 +231,8 @@ int dfhip_silu_mul_bf16(const void* gate, int64_t ld_gate, const void* up, int64
                         void* out, int64_t ld_out, int M, int D, int round_inputs_product,
                         dfhip_stream_t stream);
 
-/* fp32 flavour of the same op (fp32 configuration). D % 4 == 0. */
+/* fp32 flavour of the same op (examples/ae/up-silu-overlap.cu:75-90 without the bf16 rounding; fp32
+ * configuration). D % 4 == 0. */
 int dfhip_silu_mul_f32(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
                        void* out, int64_t ld_out, int M, int D, dfhip_stream_t stream);
 
@@ -235,8 +250,9 @@ int dfhip_rmsnorm_bf16(const void* x, const void* residual, const void* weight, 
  * convention: pairs (x[i], x[i + head_dim/2]) of every head are rotated by the
  * angle of position (row % seq_len), cos/sin tables [seq_len, head_dim/2] fp32;
  * fp32 arithmetic, one rounding.  This is model code of the host framework in
- * the reference (it reaches DynaFlow as a chain of elementwise FX nodes); here
- * one launch.  head_dim % 16 == 0. */
+ * the reference (it reaches DynaFlow as a chain of elementwise FX nodes that
+ * dynaflow/runtime/engine.py:381 runs through PyTorch; examples/ae/MOE.md:29 counts it among the
+ * "CUDA-bound" kernels of a step); here one launch.  head_dim % 16 == 0. */
 int dfhip_rope_bf16(const void* x, int64_t ld_x, void* out, int64_t ld_out, const float* cos_table,
                     const float* sin_table, int T, int heads, int head_dim, int seq_len,
                     dfhip_stream_t stream);
@@ -297,7 +313,8 @@ int dfhip_decode_attention_bf16(const void* q, int64_t ld_q, const void* k_cache
                                 dfhip_stream_t stream);
 
 /* out[N,K] = in[K,N]^T for bf16 matrices: packs a weight kept as [in, out]
- * (x @ W convention) into the [out, in] layout the GEMMs read.  K, N % 8 == 0. */
+ * (x @ W convention) into the [out, in] layout the GEMMs read.  K, N % 8 == 0.  No counterpart in the
+ * reference (torch.nn.functional.linear takes [out, in] weights as they are): a set-up helper. */
 int dfhip_transpose_bf16(const void* in, int64_t ld_in, void* out, int64_t ld_out, int K, int N,
                          dfhip_stream_t stream);
 
@@ -306,7 +323,9 @@ int dfhip_transpose_bf16(const void* in, int64_t ld_in, void* out, int64_t ld_ou
  * Per-tensor dynamic quantisation of a bf16 activation to e4m3fn in two
  * launches: (1) amax[0] = max |x| (fp32; the caller zero-fills amax[0] before
  * the launch), (2) scale[0] = max(amax, 1e-12) / 448, q = e4m3fn(x / scale[0]),
- * round-to-nearest-even, saturating at +-448. */
+ * round-to-nearest-even, saturating at +-448.  The reference ships no fp8 path of its own: these are
+ * the quantisation nodes a host framework puts in front of an fp8 `linear` (run, like every node of a
+ * sub-graph, at dynaflow/runtime/engine.py:381). */
 int dfhip_absmax_bf16(const void* x, int64_t ld, int M, int D, float* amax,
                       dfhip_stream_t stream);
 int dfhip_quant_fp8_bf16(const void* x, int64_t ld, void* q, int64_t ld_q, int M, int D,
@@ -314,13 +333,15 @@ int dfhip_quant_fp8_bf16(const void* x, int64_t ld, void* q, int64_t ld_q, int M
 
 /* silu(gate)*up in fp32 from bf16 inputs, written as bf16 to `out` (may be
  * NULL) and reduced into amax[0] = max |silu(g)*u| for the following
- * re-quantisation of the down-projection's input. */
+ * re-quantisation of the down-projection's input (the SiLU*mul of examples/ae/up-silu-overlap.cu:75-90
+ * with the absmax that a per-tensor quantisation needs). */
 int dfhip_silu_mul_absmax_bf16(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
                                void* out, int64_t ld_out, int M, int D, float* amax,
                                dfhip_stream_t stream);
 
 /* Fill `count` 32-bit words with `value` (a capture-safe replacement for
- * memset nodes, used to clear amax cells). */
+ * memset nodes, used to clear amax cells).  No counterpart in the reference (there a cudaMemset inside a
+ * captured graph is fine, dynaflow/executor/cudagraph.py:84-122 captures whatever the callable issues). */
 int dfhip_fill_u32(void* dst, uint32_t value, int64_t count, dfhip_stream_t stream);
 
 #ifdef __cplusplus
