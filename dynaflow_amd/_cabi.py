@@ -4,6 +4,10 @@ Loading is explicit and loud: there is no substitute implementation.  If the
 shared library has not been built, ``load()`` raises ``KernelLibraryMissing``
 naming the build command, and every operator that needs a kernel propagates
 that error.
+
+The reference has no kernel FFI on this path (its sub-graphs call PyTorch,
+dynaflow/runtime/engine.py:381); the callables built on this binding go where
+it keeps a sub-graph's callable (dynaflow/executor/compiler.py:69-85).
 """
 from __future__ import annotations
 

@@ -11,9 +11,12 @@ deeper), which lets a single ``Mod`` rule cut the graph:
 Tokens are flattened, ``x[T, H]`` with ``T = B * seq_len``; ``seq_len`` is a
 constructor constant, so a nano-batch (a whole number of sequences) keeps the
 layout.  Everything is plain PyTorch and also runs on the CPU; on the GPU the
-lowering pass moves the projections, SiLU*mul and RMSNorm onto the HIP
-operators, attention stays on PyTorch's fused attention kernel and RoPE on its
-elementwise kernels.
+lowering pass moves the projections, SiLU*mul, RMSNorm, RoPE and (at head_dim
+128 and sequence lengths that are multiples of 64) the causal attention onto the
+HIP operators; other attention shapes stay on PyTorch's fused attention kernel.
+
+In the reference the layer is host-model code: the decoder layer of the HF Llama
+that examples/ae/scripts/bench_hf_transformers.py:206-210 loads and traces.
 """
 from __future__ import annotations
 

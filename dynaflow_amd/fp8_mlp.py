@@ -11,6 +11,9 @@ Traced by dynamo the forward is
 linear_fp8``; ``MLPOverlapScheduler`` cuts it in front of ``silu_mul_quant_fp8``.  With ``fuse_gate_up`` the two
 projections and the SiLU*mul are one operator (``gate_up_silu_quant_fp8``) and the cut (knob
 ``fuse_silu_epilogue``) is in front of the down projection.
+
+The reference ships no fp8 model code; this block stands for the quantised MLP of a host
+framework, scheduled through the same interface (dynaflow/interface.py) as the bf16 one.
 """
 from __future__ import annotations
 

@@ -5,6 +5,11 @@ written so that dynamo traces both projections before the activation
 (``linear, linear_1, silu, mul, linear_2``); the split rule of
 ``MLPOverlapScheduler`` then yields the two sub-graphs {gate, up} and
 {silu, mul, down}.
+
+In the reference this block is host-model code (the MLP of the HF Llama that
+examples/ae/scripts/bench_hf_transformers.py:206-210 loads, whose projections
+examples/ae/scheduler/hf/nanoflow.py:30 names); its stand-alone experiment on
+the same shapes is examples/ae/up-silu-overlap.cu:266-342.
 """
 from __future__ import annotations
 

@@ -5,6 +5,11 @@ nodes traced from the ``MLPBlock`` instance becomes a sub-graph of its own (tag 
 stream), everything in front of it (embedding, attention block) is the other one.  The split is
 the balanced two-way cut at a request (sequence) boundary, the order is the staggered one, so the
 issue order is  (attn, b0) (mlp, b0) (attn, b1) (mlp, b1)  with (attn, b1) beside (mlp, b0).
+
+``Mod`` is the module-stack condition of dynaflow/matching.py:19-50; the balanced cut is the
+split policy of examples/ae/scheduler/hf/nanoflow.py:65-120, the order that of
+examples/ae/scheduler/megatron/nanoflow.py:78-102; two sub-graphs with different resource profiles
+side by side is the case examples/ae/OVERLAP.md:161-176 argues for.
 """
 from __future__ import annotations
 

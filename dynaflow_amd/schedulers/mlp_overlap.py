@@ -19,6 +19,11 @@ nano-batch i's down projection.
 Split policy: ``additional_config["num_nano_batches"]`` equal chunks (default
 ``max_num_splits``); with ``split_policy="balanced"`` the two-way balanced cut
 at a request boundary.
+
+A policy file in the shape of the reference's own (rules and hooks like
+examples/ae/scheduler/hf/nanoflow.py:46-62, streams picked from the tag like :138-146, the
+staggered order of examples/ae/scheduler/megatron/nanoflow.py:78-102); which two kinds of work
+may share the compute units follows the rule of examples/ae/OVERLAP.md:161-176.
 """
 from __future__ import annotations
 
