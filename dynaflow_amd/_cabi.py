@@ -97,6 +97,8 @@ SIGNATURES: dict[str, tuple] = {
                                           c_int, c_int, c_int, _P]),
     "dfhip_decode_attention_bf16": (c_int, [_P, c_int64, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int,
                                             c_int, c_int, ctypes.c_float, _P]),
+    "dfhip_decode_attention_append_bf16": (c_int, [_P, c_int64, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int,
+                                                   c_int, c_int, c_int, c_int, c_int, ctypes.c_float, _P]),
     "dfhip_transpose_bf16": (c_int, [_P, c_int64, _P, c_int64, c_int, c_int, _P]),
     "dfhip_absmax_bf16": (c_int, [_P, c_int64, c_int, c_int, _P, _P]),
     "dfhip_quant_fp8_bf16": (c_int, [_P, c_int64, _P, c_int64, c_int, c_int, _P, _P, _P]),

@@ -22,6 +22,16 @@ DFHIP_DEVICE f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
+// The rotation of one pair (x[i], x[i + 64]) of a head by the angle of its position: the one formula of both kernels
+// below, so that they round alike.
+// (The fused multiply-adds are spelt out: left to the compiler the two kernels could contract the expressions
+// differently.)
+DFHIP_DEVICE void rotate_pair(float lo, float hi, float c, float s, bf16_t& out_lo, bf16_t& out_hi) {
+  out_lo = static_cast<bf16_t>(__builtin_fmaf(lo, c, -(hi * s)));
+  out_hi = static_cast<bf16_t>(__builtin_fmaf(hi, c, lo * s));
+}
+DFHIP_DEVICE uint16_t bits_of(bf16_t v) { return __builtin_bit_cast(uint16_t, v); }
+
 struct KVFrags {
   bf16x8 k[2][4];   // [set][k-step]
   bf16x8 v[8];      // [dim block]
@@ -31,11 +41,19 @@ struct KVFrags {
 // MFMA row i of a score tile is mapped to position 8*(i/4) + i%4 (+4 for the second tile of the
 // chunk), so that after the two tiles lane (head = lane%16, g = lane/16) holds the scores of its
 // head for positions 8g .. 8g+7 - which is exactly the A-operand fragment of P for the P V product.
+//
+// APPEND: the workgroup first does what rope_kv_append_kernel does for its share of the token - `q` is the
+// token's row of the q / k / v product, the group's query heads are rotated in registers, the kv head's new key
+// is rotated and, with the new value, written to the caches at position lengths[t] - 1 - and then attends.  The
+// new key and value reach the wave whose chunk holds that position through LDS (its fragments are patched), not
+// through a read of what was just written.
+template <bool APPEND>
 __global__ void __launch_bounds__(DEC_THREADS)
-decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint16_t* __restrict__ kc,
-                        const uint16_t* __restrict__ vc, const int32_t* __restrict__ slots,
+decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, uint16_t* __restrict__ kc,
+                        uint16_t* __restrict__ vc, const int32_t* __restrict__ slots,
                         const int32_t* __restrict__ lengths, uint16_t* __restrict__ out, int64_t ld_out,
-                        int kv_heads, int group, int num_slots, int capacity, float scale_log2) {
+                        int kv_heads, int group, int num_slots, int capacity, float scale_log2,
+                        const float* __restrict__ cos_t, const float* __restrict__ sin_t, int table_rows) {
   // partial results of the four waves, sized by the launch for the real group (a workgroup that asks for
   // little LDS leaves room for a GEMM workgroup of the other nano-batch on the same CU)
   extern __shared__ __attribute__((aligned(16))) float combine_lds[];
@@ -52,10 +70,15 @@ decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
     for (int idx = tid; idx < group * HD; idx += DEC_THREADS) out_row[idx] = 0;
     return;
   }
+  const int pos = len - 1;                     // APPEND: the new token's position (before the clamp below)
+  const bool append = APPEND && pos < capacity;
   len = len < capacity ? len : capacity;
   const int64_t head_base = ((int64_t)slot * kv_heads + kvh) * capacity * HD;
-  const uint16_t* kbase = kc + head_base;
-  const uint16_t* vbase = vc + head_base;
+  uint16_t* kbase = kc + head_base;
+  uint16_t* vbase = vc + head_base;
+  const int trow = pos < table_rows ? pos : table_rows - 1;
+  uint16_t* const new_k = reinterpret_cast<uint16_t*>(l_lds + 4 * group);   // [HD], APPEND only
+  uint16_t* const new_v = new_k + HD;                                        // [HD]
 
   bf16x8 qf[4];
 #pragma unroll
@@ -88,6 +111,25 @@ decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
   for (int nb = 0; nb < 8; ++nb) o[nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
   auto step = [&](KVFrags& f, int c) {
+    if (APPEND && append && c == pos / CHUNK) {
+      // the chunk of the new token: its key row and value column come from LDS, whatever the loads returned
+      const int krow_pos = c * CHUNK + 8 * (hq >> 2) + (hq & 3);
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+        if (krow_pos + 4 * s == pos) {
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) f.k[s][ks] = *reinterpret_cast<const bf16x8*>(new_k + 32 * ks + 8 * g);
+        }
+      if (pos / 8 == c * (CHUNK / 8) + g) {
+#pragma unroll
+        for (int nb = 0; nb < 8; ++nb) {
+          const uint16_t v = new_v[nb * 16 + hq];
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (e == (pos & 7)) f.v[nb][e] = __builtin_bit_cast(bf16_t, v);
+        }
+      }
+    }
     if ((c + 1) * CHUNK > len) {
       // the last chunk of the sequence: positions from len on may hold anything (a cache that was never
       // written there, NaN bit patterns included) and their probability 0 would not silence a NaN in the
@@ -146,6 +188,42 @@ decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
   const int chunks = (len + CHUNK - 1) / CHUNK;
   KVFrags fa, fb;
   if (wave < chunks) load(fa, wave);
+  // (the first chunk's loads are on their way while the new token is rotated and appended)
+  if (APPEND) {
+    // the lane's fragments ks and ks + 2 hold the two halves of the pairs i = 32 ks + 8 g + e, ks = 0, 1
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int i = 32 * ks + 8 * g + e;
+        const float c = cos_t[trow * (HD / 2) + i], s = sin_t[trow * (HD / 2) + i];
+        bf16_t lo, hi;
+        rotate_pair(static_cast<float>(qf[ks][e]), static_cast<float>(qf[ks + 2][e]), c, s, lo, hi);
+        qf[ks][e] = lo;
+        qf[ks + 2][e] = hi;
+      }
+    // the kv head's new key (rotated) and value: to LDS for this workgroup, to the caches for the later steps
+    const int q_heads = kv_heads * group;
+    const uint16_t* row = q + (int64_t)t * ld_q;
+    if (tid < HD / 2) {
+      const uint16_t* k_in = row + (int64_t)(q_heads + kvh) * HD;
+      const float c = cos_t[trow * (HD / 2) + tid], s = sin_t[trow * (HD / 2) + tid];
+      bf16_t lo, hi;
+      rotate_pair(bf16_bits_to_f32(k_in[tid]), bf16_bits_to_f32(k_in[tid + 64]), c, s, lo, hi);
+      new_k[tid] = bits_of(lo);
+      new_k[tid + 64] = bits_of(hi);
+      if (append) {
+        kbase[(int64_t)pos * HD + tid] = bits_of(lo);
+        kbase[(int64_t)pos * HD + tid + 64] = bits_of(hi);
+      }
+    } else if (tid >= 64 && tid < 64 + HD) {
+      const int dim = tid - 64;
+      const uint16_t v = row[(int64_t)(q_heads + kv_heads + kvh) * HD + dim];
+      new_v[dim] = v;
+      if (append) vbase[((int64_t)(pos >> 3) * HD + dim) * 8 + (pos & 7)] = v;
+    }
+    __syncthreads();
+  }
   for (int c = wave; c < chunks; c += 8) {
     if (c + 4 < chunks) load(fb, c + 4);
     step(fa, c);
@@ -203,16 +281,16 @@ rope_kv_append_kernel(const uint16_t* __restrict__ qkv, int64_t ld_qkv, uint16_t
     const int head = idx >> 6, i = idx & 63;
     const float lo = bf16_bits_to_f32(row[head * HD + i]), hi = bf16_bits_to_f32(row[head * HD + i + 64]);
     const float c = cos_t[trow * (HD / 2) + i], s = sin_t[trow * (HD / 2) + i];
-    const uint16_t olo = static_cast<uint16_t>(f32_to_bf16_bits(lo * c - hi * s));
-    const uint16_t ohi = static_cast<uint16_t>(f32_to_bf16_bits(hi * c + lo * s));
+    bf16_t olo, ohi;
+    rotate_pair(lo, hi, c, s, olo, ohi);
     if (head < q_heads) {
       uint16_t* dst = q_out + (int64_t)t * ld_q + head * HD + i;
-      dst[0] = olo;
-      dst[64] = ohi;
+      dst[0] = bits_of(olo);
+      dst[64] = bits_of(ohi);
     } else if (cache_ok) {
       uint16_t* dst = kc + ((slot_base + (head - q_heads)) * capacity + pos) * HD + i;
-      dst[0] = olo;
-      dst[64] = ohi;
+      dst[0] = bits_of(olo);
+      dst[64] = bits_of(ohi);
     }
   }
   if (!cache_ok) return;
@@ -258,10 +336,35 @@ extern "C" int dfhip_decode_attention_bf16(const void* q, int64_t ld_q, const vo
   const float scale_log2 = scale * 1.4426950408889634f;
   const int group = q_heads / kv_heads;
   const size_t combine_bytes = (size_t)4 * group * (HD + 2) * sizeof(float);
-  hipLaunchKernelGGL(decode_attention_kernel, dim3(T * kv_heads), dim3(DEC_THREADS), combine_bytes,
+  hipLaunchKernelGGL(decode_attention_kernel<false>, dim3(T * kv_heads), dim3(DEC_THREADS), combine_bytes,
                      static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(q), ld_q,
-                     static_cast<const uint16_t*>(k_cache), static_cast<const uint16_t*>(v_cache), slots, lengths,
+                     static_cast<uint16_t*>(const_cast<void*>(k_cache)), static_cast<uint16_t*>(const_cast<void*>(v_cache)),
+                     slots, lengths, static_cast<uint16_t*>(out), ld_out, kv_heads, group, num_slots, capacity,
+                     scale_log2, nullptr, nullptr, 1);
+  return dfhip_check_launch();
+}
+
+extern "C" int dfhip_decode_attention_append_bf16(const void* qkv, int64_t ld_qkv, void* k_cache, void* v_cache,
+                                                  const int32_t* slots, const int32_t* lengths,
+                                                  const float* cos_table, const float* sin_table, void* out,
+                                                  int64_t ld_out, int T, int q_heads, int kv_heads, int head_dim,
+                                                  int num_slots, int capacity, int table_rows, float scale,
+                                                  dfhip_stream_t stream) {
+  if (!qkv || !k_cache || !v_cache || !slots || !lengths || !cos_table || !sin_table || !out)
+    return DFHIP_ERR_NULL_POINTER;
+  if (T < 1 || q_heads < 1 || kv_heads < 1 || q_heads % kv_heads != 0 || q_heads / kv_heads > MAX_GROUP ||
+      head_dim != HD || num_slots < 1 || capacity < CHUNK || capacity % CHUNK != 0 || table_rows < 1 ||
+      (int64_t)T * kv_heads >= (int64_t)1 << 31)
+    return DFHIP_ERR_BAD_SHAPE;
+  if (ld_qkv < (int64_t)(q_heads + 2 * kv_heads) * HD || ld_out < (int64_t)q_heads * HD) return DFHIP_ERR_BAD_STRIDE;
+  if (ld_qkv % 8 || !dfhip_aligned16(qkv) || !dfhip_aligned16(k_cache) || !dfhip_aligned16(v_cache))
+    return DFHIP_ERR_BAD_ALIGNMENT;
+  const int group = q_heads / kv_heads;
+  const size_t lds_bytes = (size_t)4 * group * (HD + 2) * sizeof(float) + 2 * HD * sizeof(uint16_t);
+  hipLaunchKernelGGL(decode_attention_kernel<true>, dim3(T * kv_heads), dim3(DEC_THREADS), lds_bytes,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(qkv), ld_qkv,
+                     static_cast<uint16_t*>(k_cache), static_cast<uint16_t*>(v_cache), slots, lengths,
                      static_cast<uint16_t*>(out), ld_out, kv_heads, group, num_slots, capacity,
-                     scale_log2);
+                     scale * 1.4426950408889634f, cos_table, sin_table, table_rows);
   return dfhip_check_launch();
 }

@@ -630,20 +630,13 @@ def _decode_attention_impl(qkv, k_cache, v_cache, slots, lengths, cos, sin, q_he
     slots, lengths, cos, sin = slots.contiguous(), lengths.contiguous(), cos.contiguous(), sin.contiguous()
     out = torch.empty((T, q_heads * d), dtype=qkv.dtype, device=qkv.device)
     if T > 0:
-        q_rot = torch.empty((T, q_heads * d), dtype=qkv.dtype, device=qkv.device)
-        stream = _stream()
-        rc = lib.dfhip_rope_kv_append_bf16(
-            qkv.data_ptr(), qkv.stride(0), q_rot.data_ptr(), q_heads * d, k_cache.data_ptr(), v_cache.data_ptr(),
-            slots.data_ptr(), lengths.data_ptr(), cos.data_ptr(), sin.data_ptr(), T, q_heads, kv_heads, d,
-            num_slots, capacity, cos.shape[0], stream,
+        # rotation, cache append and attention in one launch
+        rc = lib.dfhip_decode_attention_append_bf16(
+            qkv.data_ptr(), qkv.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), slots.data_ptr(),
+            lengths.data_ptr(), cos.data_ptr(), sin.data_ptr(), out.data_ptr(), q_heads * d, T, q_heads, kv_heads, d,
+            num_slots, capacity, cos.shape[0], 1.0 / math.sqrt(d), _stream(),
         )
-        _cabi.check("dfhip_rope_kv_append_bf16", rc)
-        rc = lib.dfhip_decode_attention_bf16(
-            q_rot.data_ptr(), q_heads * d, k_cache.data_ptr(), v_cache.data_ptr(), slots.data_ptr(),
-            lengths.data_ptr(), out.data_ptr(), q_heads * d, T, q_heads, kv_heads, d, num_slots, capacity,
-            1.0 / math.sqrt(d), stream,
-        )
-        _cabi.check("dfhip_decode_attention_bf16", rc)
+        _cabi.check("dfhip_decode_attention_append_bf16", rc)
     return out
 
 

@@ -287,7 +287,7 @@ int dfhip_causal_attention_bf16(const void* q, int64_t ld_q, const void* k, int6
  * with its paged cache (an FX node the schedulers treat as opaque:
  * examples/ae/scheduler/vllm/nanoflow.py:89-95 tags `unified_attention.*`
  * "attention", "no-cudagraph"); here
- * two kernels.
+ * two kernels, or one that does both.
  *
  * dfhip_rope_kv_append_bf16: qkv[T, (q_heads + 2 kv_heads) * 128] holds q, k, v
  *   of the new tokens; q and k are rotated (half-split pairs, cos/sin tables
@@ -302,7 +302,12 @@ int dfhip_causal_attention_bf16(const void* q, int64_t ld_q, const void* k, int6
  *   used, whatever they hold (uninitialised memory, NaN patterns).  A length
  *   beyond `capacity` is the caller's error and is not reported (nothing here
  *   synchronises): the append leaves the caches untouched and the token attends
- *   over the `capacity` cached positions, its own key and value not among them. */
+ *   over the `capacity` cached positions, its own key and value not among them.
+ * dfhip_decode_attention_append_bf16: both in ONE launch, same caches and same out bits as the two
+ *   calls above: every (token, kv head) workgroup rotates its query heads in registers, rotates and
+ *   appends its kv head's new key and value, and attends; the new key and value reach the products
+ *   through LDS, not through a read of what was just written.  One launch less per layer and
+ *   nano-batch of a decode step, and no q_out buffer. */
 int dfhip_rope_kv_append_bf16(const void* qkv, int64_t ld_qkv, void* q_out, int64_t ld_q, void* k_cache,
                               void* v_cache, const int32_t* slots, const int32_t* lengths,
                               const float* cos_table, const float* sin_table, int T, int q_heads, int kv_heads,
@@ -311,6 +316,11 @@ int dfhip_decode_attention_bf16(const void* q, int64_t ld_q, const void* k_cache
                                 const int32_t* slots, const int32_t* lengths, void* out, int64_t ld_out, int T,
                                 int q_heads, int kv_heads, int head_dim, int num_slots, int capacity, float scale,
                                 dfhip_stream_t stream);
+int dfhip_decode_attention_append_bf16(const void* qkv, int64_t ld_qkv, void* k_cache, void* v_cache,
+                                       const int32_t* slots, const int32_t* lengths, const float* cos_table,
+                                       const float* sin_table, void* out, int64_t ld_out, int T, int q_heads,
+                                       int kv_heads, int head_dim, int num_slots, int capacity, int table_rows,
+                                       float scale, dfhip_stream_t stream);
 
 /* out[N,K] = in[K,N]^T for bf16 matrices: packs a weight kept as [in, out]
  * (x @ W convention) into the [out, in] layout the GEMMs read.  K, N % 8 == 0.  No counterpart in the

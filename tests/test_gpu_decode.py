@@ -72,6 +72,61 @@ def test_decode_attention_against_oracle(ops, heads, kv_heads, capacity, lengths
     assert torch.equal(got_k[untouched], k_nat.double().permute(0, 2, 1, 3)[untouched])
 
 
+@pytest.mark.parametrize("heads,kv_heads,capacity,lengths", [
+    (4, 1, 32, [1, 2, 31, 32, 40]),                  # 40: beyond the capacity, nothing is appended
+    (32, 8, 256, [256, 129, 128, 127, 5, 200, 97]),
+    (16, 1, 96, [96, 95, 65, 33, 8]),
+    (3, 3, 160, [160, 1, 77, 159]),
+])
+def test_one_launch_decode_attention_has_the_bits_of_the_two_launches(heads, kv_heads, capacity, lengths):
+    """dfhip_decode_attention_append_bf16 (rotation, cache append and attention in one launch) against
+    dfhip_rope_kv_append_bf16 followed by dfhip_decode_attention_bf16 through the C ABI: the same output bits and
+    the same caches, the new position in every place a fragment can hold it, a bad slot and a length beyond the
+    capacity included."""
+    import math
+
+    from dynaflow_amd import _cabi
+    from dynaflow_amd.decode import pack_v_cache
+    from dynaflow_amd.decoder import rope_tables
+
+    lib = _cabi.load()
+    T, slots_n = len(lengths), len(lengths) + 2
+    g = torch.Generator().manual_seed(7 * capacity + heads)
+    qkv = torch.randn(T, (heads + 2 * kv_heads) * D, generator=g).bfloat16().cuda()
+    slots = torch.randperm(slots_n, generator=g)[:T].int()
+    slots[-1] = slots_n + 3 if capacity == 160 else slots[-1]       # one token with a slot out of range
+    slots = slots.cuda()
+    lens = torch.tensor(lengths, dtype=torch.int32).cuda()
+    cos, sin = (t.cuda() for t in rope_tables(capacity, D, 500000.0))
+    k0 = torch.randn(slots_n, kv_heads, capacity, D, generator=g).bfloat16()
+    v0 = pack_v_cache(torch.randn(slots_n, kv_heads, capacity, D, generator=g).bfloat16())
+    stream = torch.cuda.current_stream().cuda_stream
+    scale = 1.0 / math.sqrt(D)
+
+    k_two, v_two = k0.clone().cuda(), v0.clone().cuda()
+    q_rot = torch.empty(T, heads * D, dtype=torch.bfloat16, device="cuda")
+    out_two = torch.full((T, heads * D), 7.0, dtype=torch.bfloat16, device="cuda")
+    print(f"two launches heads={heads} kv_heads={kv_heads} capacity={capacity}", flush=True)
+    _cabi.check("dfhip_rope_kv_append_bf16", lib.dfhip_rope_kv_append_bf16(
+        qkv.data_ptr(), qkv.stride(0), q_rot.data_ptr(), heads * D, k_two.data_ptr(), v_two.data_ptr(), slots.data_ptr(),
+        lens.data_ptr(), cos.data_ptr(), sin.data_ptr(), T, heads, kv_heads, D, slots_n, capacity, cos.shape[0], stream))
+    _cabi.check("dfhip_decode_attention_bf16", lib.dfhip_decode_attention_bf16(
+        q_rot.data_ptr(), heads * D, k_two.data_ptr(), v_two.data_ptr(), slots.data_ptr(), lens.data_ptr(),
+        out_two.data_ptr(), heads * D, T, heads, kv_heads, D, slots_n, capacity, scale, stream))
+    k_one, v_one = k0.clone().cuda(), v0.clone().cuda()
+    out_one = torch.full((T, heads * D), 7.0, dtype=torch.bfloat16, device="cuda")
+    print("one launch", flush=True)
+    _cabi.check("dfhip_decode_attention_append_bf16", lib.dfhip_decode_attention_append_bf16(
+        qkv.data_ptr(), qkv.stride(0), k_one.data_ptr(), v_one.data_ptr(), slots.data_ptr(), lens.data_ptr(),
+        cos.data_ptr(), sin.data_ptr(), out_one.data_ptr(), heads * D, T, heads, kv_heads, D, slots_n, capacity,
+        cos.shape[0], scale, stream))
+    torch.cuda.synchronize()
+    assert torch.equal(k_one, k_two) and torch.equal(v_one, v_two)
+    assert not torch.equal(k_one.cpu(), k0)                       # something was appended
+    assert torch.equal(out_one, out_two)
+    assert torch.isfinite(out_one.float()).all()
+
+
 def test_decode_attention_ignores_what_lies_past_the_length(ops):
     """Caches are usually allocated uninitialised or hold recycled slots: NaN and Inf patterns in positions
     from lengths[t] on (keys and values) must not reach the output, and the result is the one a cache with
