@@ -1110,7 +1110,7 @@ int launch_walk(const void* A, int64_t lda, const void* W, const void* W2, int64
 // Decode-sized activations (a nano-batch of single-token queries): the GEMM is bound by reading W
 // once from HBM.  Tile 128 rows x 128 columns, 4 waves of 64 x 64, K in slabs of 64 through
 // a ring of four 32 KiB units (A half + W half of a slab) filled by LDS-DMA, three slabs in flight per
-// workgroup.  K is split over `split_k` workgroups per tile so that about 200 workgroups stream
+// workgroup.  K is split over `split_k` workgroups per tile so that up to 256 workgroups (one round) stream
 // different parts of W at the same time; the parts meet through the same ticket scheme as above.
 // Workgroups of one K part are neighbours (they share the A columns of that part in one XCD's L2),
 // and with more than 128 rows the row tiles of one column tile are direct neighbours: W leaves HBM
@@ -1433,12 +1433,13 @@ extern "C" int dfhip_gemm_bf16_plan_shared(int M, int N, int K, int share, int* 
   const int tiles = (int)skinny_tiles(M, N);
   const bool one_round = tiles <= 256 && (M <= 512 || (M <= SK_MAX_M && K <= 8192));
   if ((M <= SK_BM || one_round) && M >= 16 && N >= 1024 && K >= 1024) {
-    // stream W with about 192 workgroups (measured best over the 8B shapes: more parts shorten every
-    // workgroup's loop below its fixed costs), at least 8 slabs per part
-    int s = (192 + tiles / 2) / tiles;
+    // stream W with as many workgroups as fit ONE round of 256 (a second round costs more than it brings), but
+    // at least 12 slabs per part: shorter loops fall below a workgroup's fixed costs and every further part is
+    // another fp32 block written and read (measured over the 8B shapes at 128 and 256 rows, parts 2 .. 12)
+    int s = 256 / tiles;
     if (s < 1) s = 1;
     if (s > 16) s = 16;
-    while (s > 1 && K / BK < 8 * s) --s;
+    while (s > 1 && K / BK < 12 * s) --s;
     *variant = 6;
     *split_k = s;
     return DFHIP_OK;

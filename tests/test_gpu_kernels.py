@@ -422,14 +422,15 @@ def test_weight_streaming_gemm_small_shapes(ops, M, N, K):
     assert bool(((g - w_).abs() <= 2 ** -7 * w_.abs() + 2e-4 * w_.abs().max()).all())
 
 
-@pytest.mark.parametrize("M,N,K,split", [(128, 4096, 4096, 6), (100, 6144, 4096, 4), (128, 14336, 4096, 2),
-                                         (128, 4096, 14336, 6), (16, 1024, 1024, 2), (256, 4096, 4096, 3),
+@pytest.mark.parametrize("M,N,K,split", [(128, 4096, 4096, 5), (100, 6144, 4096, 5), (128, 14336, 4096, 2),
+                                         (128, 4096, 14336, 8), (16, 1024, 1024, 1), (256, 4096, 4096, 4),
                                          (192, 14336, 4096, 1), (300, 4096, 14336, 2), (512, 6144, 4096, 1),
-                                         (384, 4096, 4096, 2), (1000, 4096, 4096, 1)])
+                                         (384, 4096, 4096, 2), (1000, 4096, 4096, 1), (256, 4096, 14336, 4)])
 def test_weight_streaming_gemm_decode_shapes(ops, M, N, K, split):
     """M <= 128, and up to 512 rows (1024 with K <= 8192) while the 128 x 128 tiles fit one round of 256
     workgroups: the plan picks
-    the weight-streaming kernel and splits K so that about 200 workgroups stream W; the parts are added in a
+    the weight-streaming kernel and splits K over as many workgroups as fit one round of 256 (at least 12 slabs of K
+    per part); the parts are added in a
     fixed order, so the result is the same on every run."""
     import ctypes
 
