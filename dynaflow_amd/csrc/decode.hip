@@ -45,8 +45,10 @@ struct KVFrags {
 // APPEND: the workgroup first does what rope_kv_append_kernel does for its share of the token - `q` is the
 // token's row of the q / k / v product, the group's query heads are rotated in registers, the kv head's new key
 // is rotated and, with the new value, written to the caches at position lengths[t] - 1 - and then attends.  The
-// new key and value reach the wave whose chunk holds that position through LDS (its fragments are patched), not
-// through a read of what was just written.
+// wave whose chunks include that position does the append and keeps the new key and value in LDS for its own
+// fragments of that position, which it patches when it gets there (no read of what was just written and no
+// barrier: the wave that wrote the LDS words is the one that reads them; the other three waves only rotate their
+// copies of the query heads).
 template <bool APPEND>
 __global__ void __launch_bounds__(DEC_THREADS)
 decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, uint16_t* __restrict__ kc,
@@ -77,6 +79,7 @@ decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, uint16_t* 
   uint16_t* kbase = kc + head_base;
   uint16_t* vbase = vc + head_base;
   const int trow = pos < table_rows ? pos : table_rows - 1;
+  const uint16_t* const token_row = q + (int64_t)t * ld_q;                  // APPEND: q | k | v of the token
   uint16_t* const new_k = reinterpret_cast<uint16_t*>(l_lds + 4 * group);   // [HD], APPEND only
   uint16_t* const new_v = new_k + HD;                                        // [HD]
 
@@ -188,7 +191,7 @@ decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, uint16_t* 
   const int chunks = (len + CHUNK - 1) / CHUNK;
   KVFrags fa, fb;
   if (wave < chunks) load(fa, wave);
-  // (the first chunk's loads are on their way while the new token is rotated and appended)
+  // (the first chunk's loads are on their way while the query heads are rotated)
   if (APPEND) {
     // the lane's fragments ks and ks + 2 hold the two halves of the pairs i = 32 ks + 8 g + e, ks = 0, 1
 #pragma unroll
@@ -202,27 +205,27 @@ decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, uint16_t* 
         qf[ks][e] = lo;
         qf[ks + 2][e] = hi;
       }
-    // the kv head's new key (rotated) and value: to LDS for this workgroup, to the caches for the later steps
-    const int q_heads = kv_heads * group;
-    const uint16_t* row = q + (int64_t)t * ld_q;
-    if (tid < HD / 2) {
-      const uint16_t* k_in = row + (int64_t)(q_heads + kvh) * HD;
-      const float c = cos_t[trow * (HD / 2) + tid], s = sin_t[trow * (HD / 2) + tid];
+    // The wave whose chunks include the new position appends: lane i rotates the pair (i, i + 64) of the new key
+    // and copies two elements of the new value - to the caches for the later steps, to LDS for this wave's own
+    // fragments of that position (the same wave writes and reads them: no barrier).
+    if (append && wave == (pos / CHUNK) % 4) {
+      const int q_heads = kv_heads * group;
+      const uint16_t* k_in = token_row + (int64_t)(q_heads + kvh) * HD;
+      const uint16_t* v_in = token_row + (int64_t)(q_heads + kv_heads + kvh) * HD;
       bf16_t lo, hi;
-      rotate_pair(bf16_bits_to_f32(k_in[tid]), bf16_bits_to_f32(k_in[tid + 64]), c, s, lo, hi);
-      new_k[tid] = bits_of(lo);
-      new_k[tid + 64] = bits_of(hi);
-      if (append) {
-        kbase[(int64_t)pos * HD + tid] = bits_of(lo);
-        kbase[(int64_t)pos * HD + tid + 64] = bits_of(hi);
+      rotate_pair(bf16_bits_to_f32(k_in[lane]), bf16_bits_to_f32(k_in[lane + 64]), cos_t[trow * (HD / 2) + lane],
+                  sin_t[trow * (HD / 2) + lane], lo, hi);
+      new_k[lane] = bits_of(lo);
+      new_k[lane + 64] = bits_of(hi);
+      kbase[(int64_t)pos * HD + lane] = bits_of(lo);
+      kbase[(int64_t)pos * HD + lane + 64] = bits_of(hi);
+#pragma unroll
+      for (int d = lane; d < HD; d += 64) {
+        const uint16_t v = v_in[d];
+        new_v[d] = v;
+        vbase[((int64_t)(pos >> 3) * HD + d) * 8 + (pos & 7)] = v;
       }
-    } else if (tid >= 64 && tid < 64 + HD) {
-      const int dim = tid - 64;
-      const uint16_t v = row[(int64_t)(q_heads + kv_heads + kvh) * HD + dim];
-      new_v[dim] = v;
-      if (append) vbase[((int64_t)(pos >> 3) * HD + dim) * 8 + (pos & 7)] = v;
     }
-    __syncthreads();
   }
   for (int c = wave; c < chunks; c += 8) {
     if (c + 4 < chunks) load(fb, c + 4);
