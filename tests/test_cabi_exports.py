@@ -58,6 +58,13 @@ def test_argument_checks_run_before_any_launch():
     assert lib.dfhip_gemm_bf16_nt_splitk_static(16, 4096, 16, 4096, 16, 4096, 4096, 4096, 4096, 2, None) == -8
     assert lib.dfhip_gemm_bf16_nt_splitk_static(None, 4096, 16, 4096, 16, 4096, 4096, 4096, 4096, 2, None) == -1
     assert lib.dfhip_gemm_bf16_nt_splitk_static(16, 4096, 16, 4096, 16, 4096, 256, 256, 4096, 17, None) == -7
+    # decode attention with the append in the same launch: pointers, head grouping, capacity, row stride, alignment
+    one = lib.dfhip_decode_attention_append_bf16
+    assert one(None, 768, 16, 16, 16, 16, 16, 16, 16, 512, 1, 4, 1, 128, 1, 32, 32, 0.1, None) == -1
+    assert one(16, 768, 16, 16, 16, 16, 16, 16, 16, 512, 1, 4, 3, 128, 1, 32, 32, 0.1, None) == -2      # 4 % 3
+    assert one(16, 768, 16, 16, 16, 16, 16, 16, 16, 512, 1, 4, 1, 128, 1, 48, 32, 0.1, None) == -2      # capacity % 32
+    assert one(16, 512, 16, 16, 16, 16, 16, 16, 16, 512, 1, 4, 1, 128, 1, 32, 32, 0.1, None) == -3      # row too short
+    assert one(8, 768, 16, 16, 16, 16, 16, 16, 16, 512, 1, 4, 1, 128, 1, 32, 32, 0.1, None) == -4       # alignment
     assert b"scratch" in lib.dfhip_status_string(-8)
 
 
