@@ -545,6 +545,13 @@ def decode_config(torch, steps, warmup, layers=32):
                                 ("overlapped_whole_graph", {"whole_graph": True}, "whole"),
                                 ("stream_per_nano_batch_whole_graph",
                                  {"streams": "by_nano_batch", "whole_graph": True}, "whole"),
+                                # the same two modes with the kernels planned for two launches that share the GPU
+                                # (knob side_by_side: the weight-streaming GEMMs split K over half as many
+                                # workgroups and move half as many fp32 blocks; another order of additions)
+                                ("stream_per_nano_batch_planned_for_two_sub_graph_replay",
+                                 {"streams": "by_nano_batch", "side_by_side": 2}, True),
+                                ("stream_per_nano_batch_planned_for_two_whole_graph",
+                                 {"streams": "by_nano_batch", "side_by_side": 2, "whole_graph": True}, "whole"),
                                 ("unsplit_sub_graph_replay", {"min_nano_split_tokens": 1 << 30}, True)):
         extra = {"min_nano_split_tokens": 1, "dump_graph": False, "max_tokens": seqs, "fuse_silu_epilogue": True,
                  **EXTRA_KNOBS}

@@ -1436,7 +1436,7 @@ extern "C" int dfhip_gemm_bf16_plan_shared(int M, int N, int K, int share, int* 
     // stream W with as many workgroups as fit ONE round of 256 (a second round costs more than it brings), but
     // at least 12 slabs per part: shorter loops fall below a workgroup's fixed costs and every further part is
     // another fp32 block written and read (measured over the 8B shapes at 128 and 256 rows, parts 2 .. 12)
-    int s = 256 / tiles;
+    int s = 256 / (tiles * share);            // launches that run side by side take the round together
     if (s < 1) s = 1;
     if (s > 16) s = 16;
     while (s > 1 && K / BK < 12 * s) --s;

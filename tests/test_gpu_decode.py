@@ -317,23 +317,26 @@ def test_decode_attention_under_graph_capture(ops):
     assert torch.equal(out, want) and not torch.equal(out, eager)
 
 
-@pytest.mark.parametrize("streams", ["by_kind", "by_nano_batch"])
-def test_decode_schedule_with_sub_graph_replay(streams):
+@pytest.mark.parametrize("streams,share", [("by_kind", 1), ("by_nano_batch", 1), ("by_nano_batch", 2)])
+def test_decode_schedule_with_sub_graph_replay(streams, share):
     """Per-sub-graph graphs (the reference's mechanism) on the decode model at shapes where the projections
     run on the weight-streaming kernel with K split: capture in a dry-run at the nano-batch size, then the
     scheduled forward replays the graphs; every replay equals the eager two-stream result - with the streams
-    chosen by sub-graph kind (attention / MLP) and with one stream per nano-batch."""
+    chosen by sub-graph kind (attention / MLP), with one stream per nano-batch, and with the kernels planned
+    for two launches that share the GPU (knob side_by_side: K split over fewer workgroups)."""
     T = 32
     over = dict(layers=2, hidden=1024, heads=8, kv_heads=2, inter=2048)
     print("decode sub-graph replay: eager model", flush=True)
-    manager, compiled, dev, host, model, inputs, cm = build_decode(T, whole_graph=False, **over)
+    manager, compiled, dev, host, model, inputs, cm = build_decode(T, whole_graph=False,
+                                                                   knobs={"side_by_side": share}, **over)
     with torch.no_grad():
         manager.prepare(T, [1] * T)
         eager = compiled(*dev).clone()
         torch.cuda.synchronize()
     print("decode sub-graph replay: graph model", flush=True)
     manager, compiled, dev, host2, model2, _, _ = build_decode(T, whole_graph=False, sub_graphs=True,
-                                                               knobs={"streams": streams}, **over)
+                                                               knobs={"streams": streams, "side_by_side": share},
+                                                               **over)
     half = T // 2
     with torch.no_grad():
         print("decode sub-graph replay: dry-run capture", flush=True)

@@ -232,6 +232,9 @@ def test_side_by_side_option_and_the_plan_for_shared_launches():
     assert plan(2048, 4096, 14336, 2) == (0, 1)
     assert plan(1024, 4096, 14336, 2) == (0, 2)          # 64 tiles, twice: still two parts each
     assert plan(2048, 14336, 4096, 1) == plan(2048, 14336, 4096, 2) == (5, 1)
-    assert plan(128, 4096, 4096, 1) == plan(128, 4096, 4096, 2) and plan(128, 4096, 4096, 2)[0] == 6
+    # the weight-streaming kernel: one round of workgroups for all the launches that share the GPU
+    assert plan(128, 4096, 4096, 1) == (6, 5) and plan(128, 4096, 4096, 2) == (6, 4)
+    assert plan(128, 4096, 14336, 1) == (6, 8) and plan(128, 4096, 14336, 2) == (6, 4)
+    assert plan(128, 6144, 4096, 2) == (6, 2) and plan(128, 14336, 4096, 2) == (6, 1)
     v, k = ctypes.c_int(), ctypes.c_int()
     assert lib.dfhip_gemm_bf16_plan_shared(2048, 4096, 14336, 0, ctypes.byref(v), ctypes.byref(k)) == -7
