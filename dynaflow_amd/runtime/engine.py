@@ -342,7 +342,12 @@ class DynaFlowEngine:
                 and _is_symbolic(example.shape[0])
                 and split_config.use_cudagraph
             ):
-                buf = self.input_buffers[0][idx]
+                buf = self.input_buffers[0].get(idx)
+                if buf is None:
+                    raise RuntimeError(
+                        "static input buffer missing: graph replay of an unsplit batch needs a dry-run with "
+                        "use_cudagraph at this size first"
+                    )
                 buf[:padded].copy_(args[idx])
                 call_args[idx] = buf[:padded]
         handle = OperatorHandle(

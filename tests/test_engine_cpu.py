@@ -106,6 +106,14 @@ def test_single_batch_takes_fast_path_and_bypasses_scheduler(host_device):
     torch.testing.assert_close(y, model(x), rtol=0, atol=0)
 
 
+def test_single_batch_graph_replay_without_a_capturing_dry_run_is_refused(host_device):
+    cfg = make_config(2, min_nano_split_tokens=1000)
+    model, manager, compiled, x = compile_mlp(cfg)
+    manager.prepare(64, [64], use_cudagraph=True)
+    with torch.no_grad(), pytest.raises(RuntimeError, match="static input buffer missing"):
+        compiled(x)
+
+
 def test_single_batch_through_scheduler_when_fallback_disallowed(host_device):
     cfg = make_config(2, min_nano_split_tokens=1000)
     model, manager, compiled, x = compile_mlp(cfg)
