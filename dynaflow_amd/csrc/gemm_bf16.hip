@@ -1115,7 +1115,10 @@ int launch_walk(const void* A, int64_t lda, const void* W, const void* W2, int64
 // Workgroups of one K part are neighbours (they share the A columns of that part in one XCD's L2),
 // and with more than 128 rows the row tiles of one column tile are direct neighbours: W leaves HBM
 // once and the other row tiles find it in that XCD's L2.
+// (a ring of five units, one more slab in flight, measured no faster on any decode shape)
 constexpr int SK_BM = 128, SK_BN = 128, SK_UNITS = 4, SK_UNIT = 32768, SK_LDS = SK_UNITS * SK_UNIT;
+constexpr int SK_AHEAD = SK_UNITS - 1;          // slabs issued ahead of the one being multiplied
+constexpr int SK_FLIGHT = (SK_AHEAD - 2) * 8;   // DMA instructions of a wave that may still be in flight at a barrier
 constexpr int SK_MAX_M = 1024;
 
 // FUSED: C[M, N] = silu(A W^T) * (A W2^T) (gate and up weights, N = the intermediate size, K not split):
@@ -1193,14 +1196,13 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
 #pragma unroll
     for (int j = 0; j < 2; ++j) fw[slot][j] = *reinterpret_cast<const bf16x8*>(u + w_lane + j * 4096 + koff[ks]);
   };
-  issue(0, 0);
-  issue(1, 1);
-  issue(2, 2);
-  wait_vmcnt<8>();           // slabs 0 and 1 have landed
+#pragma unroll
+  for (int u = 0; u < SK_AHEAD; ++u) issue(u, u);
+  wait_vmcnt<SK_FLIGHT>();   // slabs 0 and 1 have landed
   workgroup_barrier();
   read_frags(0, 0, 0);
   for (int kt = 0; kt < KT; ++kt) {
-    issue(kt + 3, (kt + 3) % SK_UNITS);   // into the unit of slab kt-1: everybody passed the barrier after it
+    issue(kt + SK_AHEAD, (kt + SK_AHEAD) % SK_UNITS);   // into the unit of slab kt-1: everybody passed the barrier after it
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       const int slot = ks & 1;
@@ -1214,7 +1216,7 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
       DFHIP_PIN;
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // every read of slab kt (and the prefetch) has returned
-    wait_vmcnt<8>();         // slab kt+2 has landed; only slab kt+3 may be in flight
+    wait_vmcnt<SK_FLIGHT>();   // slab kt+2 has landed; only the slabs after it may be in flight
     workgroup_barrier();
   }
   wait_vmcnt<0>();

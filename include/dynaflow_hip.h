@@ -307,7 +307,10 @@ int dfhip_causal_attention_bf16(const void* q, int64_t ld_q, const void* k, int6
  *   calls above: every (token, kv head) workgroup rotates its query heads in registers, rotates and
  *   appends its kv head's new key and value, and attends; the new key and value reach the products
  *   through LDS, not through a read of what was just written.  One launch less per layer and
- *   nano-batch of a decode step, and no q_out buffer. */
+ *   nano-batch of a decode step, and no q_out buffer.
+ * The tokens of one call (and of calls that run at the same time) name distinct slots: a decode
+ *   step has one new token per sequence, and two tokens of one slot would append to and read one
+ *   cache concurrently. */
 int dfhip_rope_kv_append_bf16(const void* qkv, int64_t ld_qkv, void* q_out, int64_t ld_q, void* k_cache,
                               void* v_cache, const int32_t* slots, const int32_t* lengths,
                               const float* cos_table, const float* sin_table, int T, int q_heads, int kv_heads,
