@@ -1336,6 +1336,141 @@ gemm_bf16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restri
   }
 }
 
+// The fused launch with twice the columns per workgroup: 128 rows x 128 outputs (128 gate rows and 128 up rows of
+// W per slab), 4 waves of 64 rows x 64 outputs (two gate and two up blocks of 32 rows each).  Half as many
+// workgroups move half as many activation bytes through LDS per weight byte and meet at half as many barriers;
+// a unit of the ring is A 16 KiB | W 32 KiB and three of them fit, so a slab's first fragments are read after the
+// barrier that follows its landing (no read ahead across slabs) and two slabs are in flight meanwhile.  For two
+// launches that share the GPU (2 x 112 workgroups at 14336 outputs: one round together) and for 129 .. 256 rows.
+// Same instruction and same order of K as gemm_bf16_skinny_kernel<true>: the same bits.
+constexpr int SKW_BN = 128, SKW_UNIT = 49152, SKW_UNITS = 3, SKW_LDS = SKW_UNITS * SKW_UNIT;
+
+__global__ void __launch_bounds__(RTHREADS)
+gemm_bf16_skinny_wide_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
+                             const uint16_t* __restrict__ W2, uint16_t* __restrict__ C, int M, int N, int K,
+                             int64_t lda, int64_t ldw, int64_t ldc, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave & 1, wave_n = wave >> 1;
+  const int tile = remap_xcd(blockIdx.x, tiles_m * tiles_n);   // column tile major, row tile minor
+  const int tile_n = tile / tiles_m;
+  const int m0 = (tile - tile_n * tiles_m) * SK_BM;
+  const int n0 = tile_n * SKW_BN;
+  const int KT = K / BK;
+
+  // DMA: the A part is 128 rows x 128 bytes = 16 instructions of 8 rows (4 per wave), the W part 256 rows = 32
+  // instructions (8 per wave); W row r of the unit: wave column r / 128, (gate, up) = (r / 64) % 2, output r % 64
+  const uint8_t* a_src[4];
+  const uint8_t* w_src[8];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int row = (wave * 4 + t) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    const int ar = m0 + row < M ? m0 + row : M - 1;
+    a_src[t] = reinterpret_cast<const uint8_t*>(A + (int64_t)ar * lda + chunk * 8);
+  }
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    const int row = (wave * 8 + t) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    int wr = n0 + (row >> 7) * 64 + (row & 63);
+    wr = wr < N ? wr : N - 1;
+    w_src[t] = reinterpret_cast<const uint8_t*>((((row >> 6) & 1) ? W2 : W) + (int64_t)wr * ldw + chunk * 8);
+  }
+  auto issue = [&](int slab, int unit) {
+    const int64_t off = (int64_t)(slab < KT ? slab : KT - 1) * (BK * 2);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) dma16(unit * SKW_UNIT + (wave * 4 + t) * 1024, a_src[t] + off);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) dma16(unit * SKW_UNIT + 16384 + (wave * 8 + t) * 1024, w_src[t] + off);
+  };
+
+  const int frow = lane & 31, fhalf = lane >> 5, fswz = (frow >> 1) & 7;
+  int koff[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) koff[ks] = ((2 * ks + fhalf) ^ fswz) * 16;
+  const int a_lane = (wave_m * 64 + frow) * 128, w_lane = 16384 + (wave_n * 128 + frow) * 128;
+
+  f32x16 acc[2][4];   // [row block][gate 0, gate 1, up 0, up 1]
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  bf16x8 fa[2][2], fw[2][4];
+  auto read_frags = [&](int unit, int ks, int slot) {
+    const uint8_t* u = smem + unit * SKW_UNIT;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) fa[slot][i] = *reinterpret_cast<const bf16x8*>(u + a_lane + i * 4096 + koff[ks]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) fw[slot][j] = *reinterpret_cast<const bf16x8*>(u + w_lane + j * 4096 + koff[ks]);
+  };
+  issue(0, 0);
+  issue(1, 1);
+  wait_vmcnt<12>();          // slab 0 has landed
+  workgroup_barrier();
+  int unit = 0;
+  for (int kt = 0; kt < KT; ++kt) {
+    read_frags(unit, 0, 0);
+    const int free_unit = unit == 0 ? SKW_UNITS - 1 : unit - 1;   // slab kt-1: everybody passed the barrier after it
+    issue(kt + 2, free_unit);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int slot = ks & 1;
+      if (ks < 3) read_frags(unit, ks + 1, slot ^ 1);
+      DFHIP_PIN;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
+      DFHIP_PIN;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // every read of slab kt has returned
+    wait_vmcnt<12>();        // slab kt+1 has landed; only slab kt+2 may be in flight
+    workgroup_barrier();
+    unit = unit == SKW_UNITS - 1 ? 0 : unit + 1;
+  }
+  wait_vmcnt<0>();
+  workgroup_barrier();
+
+  // the roundings of the separate kernels (bf16 projections, bf16 silu, bf16 product); 64 rows x 64 outputs per
+  // wave are parked in LDS (144-byte rows) and leave as whole 128-byte row pieces
+  constexpr int PROW = 144;
+  uint8_t* park = smem + wave * (64 * PROW);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float p[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float gt = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][jj][4 * g + e]));
+          const float ut = bf16_bits_to_f32(f32_to_bf16_bits(acc[i][2 + jj][4 * g + e]));
+          p[e] = bf16_bits_to_f32(f32_to_bf16_bits(silu_fast(gt))) * ut;
+        }
+        u32x2 v;
+        v[0] = pack2_bf16(p[0], p[1]);
+        v[1] = pack2_bf16(p[2], p[3]);
+        *reinterpret_cast<u32x2*>(park + (i * 32 + frow) * PROW + (jj * 32 + g * 8 + fhalf * 4) * 2) = v;
+      }
+  DFHIP_PIN;
+  const int m_base = m0 + wave_m * 64, n_base = n0 + wave_n * 64;
+#pragma unroll 4
+  for (int p = 0; p < 8; ++p) {
+    const int id = p * 64 + lane;
+    const int row = id >> 3, c = id & 7;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * PROW + c * 16);
+    const int m = m_base + row, n = n_base + c * 8;
+    if (m < M && n < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(C + (int64_t)m * ldc + n));
+  }
+}
+
 size_t skinny_tiles(int M, int N) { return (size_t)((M + SK_BM - 1) / SK_BM) * ((N + SK_BN - 1) / SK_BN); }
 size_t skinny_counter_bytes(int M, int N) { return counter_area(skinny_tiles(M, N)); }
 
@@ -1356,6 +1491,21 @@ int launch_skinny(const void* A, int64_t lda, const void* W, const void* W2, int
                      static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W),
                      static_cast<const uint16_t*>(W2), static_cast<uint16_t*>(C), M, N, K, lda, ldw, ldc, tiles_m,
                      tiles_n, split_k, partials, arrivals);
+  return dfhip_check_launch();
+}
+
+int launch_skinny_wide(const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw, void* C, int64_t ldc,
+                       int M, int N, int K, hipStream_t stream) {
+  if (M > SK_MAX_M || K / BK < 2) return DFHIP_ERR_BAD_SHAPE;
+  auto kernel = gemm_bf16_skinny_wide_kernel;
+  static std::atomic<uint64_t> lds_opted_in{0};
+  if (int rc = dfhip_opt_in_lds(reinterpret_cast<const void*>(kernel), SKW_LDS, lds_opted_in)) return rc;
+  const int tiles_m = (M + SK_BM - 1) / SK_BM;
+  const int tiles_n = (N + SKW_BN - 1) / SKW_BN;
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(RTHREADS), SKW_LDS, stream,
+                     static_cast<const uint16_t*>(A), static_cast<const uint16_t*>(W),
+                     static_cast<const uint16_t*>(W2), static_cast<uint16_t*>(C), M, N, K, lda, ldw, ldc, tiles_m,
+                     tiles_n);
   return dfhip_check_launch();
 }
 
@@ -1515,9 +1665,17 @@ extern "C" int dfhip_gemm_bf16_gate_up_silu_shared(const void* A, int64_t lda, c
   if (share < 1 || share > 16) return DFHIP_ERR_BAD_ARGUMENT;
   if (int rc = check_args(A, lda, W_gate, ldw, Out, ldo, M, I, K)) return rc;
   if (!dfhip_aligned16(W_up)) return DFHIP_ERR_BAD_ALIGNMENT;
-  if (M <= 2 * SK_BM && I >= 1024 && K >= 1024)   // decode-sized activations: stream both weights once
+  if (M <= 2 * SK_BM && I >= 1024 && K >= 1024) {   // decode-sized activations: stream both weights once
+    // 128 outputs per workgroup when the launches that run side by side, or the two row tiles of 129 .. 256
+    // rows, then still give every compute unit a workgroup's worth of the round; 64 outputs otherwise
+    // (8B shape, us: a pair of 128-row launches on two streams 99.5 -> 88, one 256-row launch 88.6 -> 75.9, but a
+    // lone 128-row launch 55 -> 71 with its 112 workgroups)
+    const int64_t wide = (int64_t)((M + SK_BM - 1) / SK_BM) * ((I + SKW_BN - 1) / SKW_BN) * share;
+    if (wide >= 192)
+      return launch_skinny_wide(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, static_cast<hipStream_t>(stream));
     return launch_skinny<true>(A, lda, W_gate, W_up, ldw, Out, ldo, M, I, K, 1, nullptr,
                                static_cast<hipStream_t>(stream));
+  }
   // the 256 x (112 + 112) tile when it fills the rounds of 256 workgroups clearly better than the 256 x (128 + 128)
   // one, which moves fewer bytes through LDS per flop; launches that run side by side take their rounds together
   // (two launches of the 8B shape at 2048 rows: 2 x 896 square tiles are exactly 7 rounds)

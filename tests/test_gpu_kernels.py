@@ -347,6 +347,27 @@ def test_gate_up_silu_fused_epilogue(ops, M, I, K):
     assert bool(((g32 - w32).abs() <= 2 ** -5 * w32.abs() + 2e-3 * w32.abs().max()).all())
 
 
+@pytest.mark.parametrize("M,I,K,share", [(128, 14336, 4096, 2), (100, 14336, 4096, 2), (1, 14336, 4096, 2),
+                                         (128, 1088, 1024, 16), (77, 3000, 2048, 16), (256, 14336, 4096, 1),
+                                         (200, 14336, 4096, 1), (129, 28672, 8192, 1)])
+def test_weight_streaming_gate_up_silu_wide_tile_has_the_bits_of_the_narrow_one(ops, M, I, K, share):
+    """Decode-sized gate/up/SiLU launches take 128 outputs per workgroup instead of 64 when the launches that run
+    side by side (`share`), or the two row tiles of 129 .. 256 rows, still make at least 192 workgroups: the same
+    instruction over K in the same order, so the same bits as the narrow tile - checked against launches of at
+    most 128 rows planned alone (which take the narrow tile unless they have 192 column tiles of their own, as
+    with 28672 outputs) and against the separate operators.
+    Ragged rows and outputs (I = 1088, 3000 are no multiples of 128) included."""
+    x = randn((M, K), 44).bfloat16().cuda()
+    wg = randn((I, K), 45, 0.02).bfloat16().cuda()
+    wu = randn((I, K), 46, 0.02).bfloat16().cuda()
+    with ops.launch_options(side_by_side=share):
+        got = ops.gate_up_silu(x, wg, wu)
+    narrow = torch.cat([ops.gate_up_silu(x[lo:lo + 128].contiguous(), wg, wu) for lo in range(0, M, 128)])
+    assert torch.equal(got, narrow)
+    separate = ops.silu_mul(ops.linear_variant(x, wg, -2), ops.linear_variant(x, wu, -2), True)
+    assert torch.equal(got, separate)
+
+
 def test_plan_prefers_224_wide_tiles_for_llama_intermediate_size(ops):
     import ctypes
 
