@@ -301,6 +301,63 @@ def decode_kernels(torch, ops, iters):
     }
 
 
+def decode_projections(torch, ops, iters):
+    """The four projections of a decode layer at 128 rows (one nano-batch), weights rotated over several copies so
+    that they come from HBM as in a 32-layer model; every case is a captured graph of four launches (or pairs):
+    one launch alone, the two nano-batches' launches side by side on two streams over the same weights (planned
+    alone and planned for two), and one launch over all 256 rows.  us per launch or pair."""
+    H, I, rows = HIDDEN, INTER, 128
+    gen = torch.Generator(device="cuda").manual_seed(6)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+
+    def replayed(body):
+        body()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            body()
+        best = min(time_kernel(torch, graph.replay, iters) for _ in range(3))
+        return round(best * 1e3 / 4, 1)
+
+    out = {}
+    for name, n, k, fused in (("qkv", 6144, H, False), ("o", H, H, False), ("gate_up_silu", I, H, True),
+                              ("down", H, I, False)):
+        xs = [torch.randn(rows, k, generator=gen, device="cuda").bfloat16() for _ in range(2)]
+        both = torch.cat(xs)
+        copies = 4 if fused else 8
+        ws = [(torch.randn(n, k, generator=gen, device="cuda") * 0.02).bfloat16() for _ in range(copies)]
+        call = (lambda x, i: ops.gate_up_silu(x, ws[i], ws[(i + 1) % copies])) if fused else \
+               (lambda x, i: ops.linear(x, ws[i]))
+
+        def alone():
+            for it in range(4):
+                call(xs[0], it)
+
+        def whole():
+            for it in range(4):
+                call(both, it)
+
+        def pairs(share):
+            def body():
+                for it in range(4):
+                    here = torch.cuda.current_stream()
+                    for stream in streams:
+                        stream.wait_stream(here)
+                    with ops.launch_options(side_by_side=share):
+                        for x, stream in zip(xs, streams):
+                            with torch.cuda.stream(stream):
+                                call(x, it)
+                    for stream in streams:
+                        here.wait_stream(stream)
+            return body
+
+        out[name] = {"one_launch_128_rows_us": replayed(alone), "pair_planned_alone_us": replayed(pairs(1)),
+                     "pair_planned_for_two_us": replayed(pairs(2)), "one_launch_256_rows_us": replayed(whole),
+                     "weight_bytes": (2 if fused else 1) * n * k * 2}
+        del ws
+    return out
+
+
 def prefill_attention_kernels(torch, ops, iters):
     """Causal grouped-query attention of one prefill nano-batch.  Algorithmic work: the causal half of the
     two products, 2 * B * heads * S * S * d FLOP."""
@@ -697,7 +754,9 @@ def main() -> int:
         print(json.dumps(decode_config(torch, max(5, args.steps // 5), max(3, args.warmup // 5))))
         return 0
     if args.decode_kernels:
-        print(json.dumps(decode_kernels(torch, ops, max(20, args.steps))))
+        line = decode_kernels(torch, ops, max(20, args.steps))
+        line["projections"] = decode_projections(torch, ops, max(20, args.steps))
+        print(json.dumps(line))
         return 0
     if args.prefill_attention_kernels:
         print(json.dumps(prefill_attention_kernels(torch, ops, max(20, args.steps))))
