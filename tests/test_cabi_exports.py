@@ -97,3 +97,32 @@ def test_header_is_plain_c_and_cpp():
         pytest.skip("no host compiler")
     subprocess.run([gcc, "-fsyntax-only", "-x", "c", "-std=c99", "-Wall", "-Werror", "-pedantic", HEADER], check=True)
     subprocess.run([gpp, "-fsyntax-only", "-x", "c++", "-std=c++11", "-Wall", "-Werror", HEADER], check=True)
+
+
+def test_the_product_never_imports_the_oracle():
+    """The oracle is test infrastructure: nothing in the package may import it, and the bench only inside its
+    CPU leg (`cpu_baseline`), the smoke test only inside `smoke`."""
+    import ast
+    import pathlib
+
+    root = pathlib.Path(__file__).resolve().parents[1]
+
+    def oracle_imports(tree):
+        found = []
+        for node in ast.walk(tree):
+            if isinstance(node, ast.Import):
+                found += [node for a in node.names if a.name.split(".")[0] == "oracle"]
+            elif isinstance(node, ast.ImportFrom) and (node.module or "").split(".")[0] == "oracle":
+                found.append(node)
+        return found
+
+    for path in (root / "dynaflow_amd").rglob("*.py"):
+        assert not oracle_imports(ast.parse(path.read_text())), f"{path} imports the oracle"
+    for name, allowed in (("bench.py", "cpu_baseline"), ("__graft_entry__.py", "smoke")):
+        tree = ast.parse((root / name).read_text())
+        inside = set()
+        for node in ast.walk(tree):
+            if isinstance(node, ast.FunctionDef) and node.name == allowed:
+                inside = {id(n) for n in oracle_imports(node)}
+        assert inside, f"{name}: {allowed} was expected to use the oracle"
+        assert {id(n) for n in oracle_imports(tree)} == inside, f"{name} imports the oracle outside {allowed}"
