@@ -97,15 +97,18 @@ decode_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, uint16_t* 
   const uint16_t* k_lane = kbase + (int64_t)krow * HD + 8 * g;
   const uint16_t* v_lane = vbase + ((int64_t)g * HD + hq) * 8;
 
+  // every cached element is read once per step and by nobody else: non-temporal loads, which do not displace
+  // what the caches hold for the kernels that run beside this one (128 sequences x 2048 positions: 187 -> 158 us)
   auto load = [&](KVFrags& f, int chunk) {
     const uint16_t* kp = k_lane + (int64_t)chunk * (CHUNK * HD);
     const uint16_t* vp = v_lane + (int64_t)chunk * (CHUNK * HD);
 #pragma unroll
     for (int s = 0; s < 2; ++s)
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) f.k[s][ks] = *reinterpret_cast<const bf16x8*>(kp + s * 4 * HD + 32 * ks);
+      for (int ks = 0; ks < 4; ++ks)
+        f.k[s][ks] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(kp + s * 4 * HD + 32 * ks));
 #pragma unroll
-    for (int nb = 0; nb < 8; ++nb) f.v[nb] = *reinterpret_cast<const bf16x8*>(vp + nb * 16 * 8);
+    for (int nb = 0; nb < 8; ++nb) f.v[nb] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(vp + nb * 16 * 8));
   };
 
   float m = -INFINITY, l = 0.0f;
