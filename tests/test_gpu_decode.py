@@ -72,6 +72,42 @@ def test_decode_attention_against_oracle(ops, heads, kv_heads, capacity, lengths
     assert torch.equal(got_k[untouched], k_nat.double().permute(0, 2, 1, 3)[untouched])
 
 
+def test_decode_attention_over_consecutive_steps_reads_what_the_previous_launch_appended(ops):
+    """Four launches in a row on the same caches, every sequence one position further each time (crossing chunk
+    boundaries of 32 and 8 positions): a launch attends over the keys and values that the launches before it
+    appended - written by ordinary stores, read back by the next kernel's non-temporal loads."""
+    from dynaflow_amd.decode import pack_v_cache
+    from dynaflow_amd.decoder import rope_tables
+
+    heads, kv_heads, capacity, start = 8, 2, 96, [1, 30, 31, 62, 7]
+    T = len(start)
+    g = torch.Generator().manual_seed(77)
+    k_nat = torch.randn(T, kv_heads, capacity, D, generator=g).bfloat16()
+    v_nat = torch.randn(T, kv_heads, capacity, D, generator=g).bfloat16()
+    cos, sin = rope_tables(capacity, D, 500000.0)
+    k_cache, v_cache = k_nat.cuda(), pack_v_cache(v_nat).cuda()
+    kc, vc = k_nat.double().permute(0, 2, 1, 3).contiguous(), v_nat.double().permute(0, 2, 1, 3).contiguous()
+    slots = torch.arange(T, dtype=torch.int32)
+    for step in range(4):
+        lens = torch.tensor([L + step for L in start], dtype=torch.int32)
+        qkv = torch.randn(T, (heads + 2 * kv_heads) * D, generator=g).bfloat16()
+        out = ops.decode_attention(qkv.cuda(), k_cache, v_cache, slots.cuda(), lens.cuda(), cos.cuda(), sin.cuda(),
+                                   heads, kv_heads)
+        pos = lens.long() - 1
+        q = ref.rope_at(qkv[:, : heads * D].double().view(T, heads, D), pos, 500000.0)
+        k_new = ref.rope_at(qkv[:, heads * D:(heads + kv_heads) * D].double().view(T, kv_heads, D), pos, 500000.0)
+        v_new = qkv[:, (heads + kv_heads) * D:].double().view(T, kv_heads, D)
+        for t in range(T):
+            L = int(lens[t])
+            # what the kernel left in the cache: the rotated key rounded to bf16, the value as it came
+            kc[t, L - 1], vc[t, L - 1] = k_new[t].bfloat16().double(), v_new[t]
+            want = ref.attend(q[t], kc[t, :L], vc[t, :L]).reshape(-1)
+            assert rel_err(out[t].float(), want) < TOL_BF16, (step, t, L)
+    got_k, got_v = natural(k_cache, v_cache)
+    assert (got_k - kc).abs().max() <= 2 ** -7 * kc.abs().max()
+    assert torch.equal(got_v, vc)
+
+
 @pytest.mark.parametrize("heads,kv_heads,capacity,lengths", [
     (4, 1, 32, [1, 2, 31, 32, 40]),                  # 40: beyond the capacity, nothing is appended
     (32, 8, 256, [256, 129, 128, 127, 5, 200, 97]),
