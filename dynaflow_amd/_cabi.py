@@ -66,6 +66,7 @@ SIGNATURES: dict[str, tuple] = {
         c_int,
         [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, c_int, _P, c_size_t, _P],
     ),
+    "dfhip_gemm_bf16_splitk_work": (c_int, [c_int, c_int, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
     "dfhip_gemm_bf16_nt_splitk_static": (
         c_int,
         [_P, c_int64, _P, c_int64, _P, c_int64, c_int, c_int, c_int, c_int, _P],

@@ -50,17 +50,27 @@ DFHIP_DEVICE float max3(float a, float b, float c) {
 // registers, where the softmax reads it with ordinary instructions, and the Q fragment - which is only ever an MFMA
 // operand - in ACCUMULATION registers.  Left to the compiler the score tiles sit in accumulation registers and
 // every score costs a v_accvgpr_read_b32, which beside running MFMAs takes about three times as long as an
-// ordinary vector instruction (take-it-out timing).  The compiler does not know that these are MFMAs: a result is
-// first read two or more MFMAs (64 cycles) after the last product into it, which covers the 11 wait states of an
-// 8-pass MFMA; the accumulating form reads exactly the registers it writes, the one dependent sequence that the
-// matrix pipe forwards by itself.
+// ordinary vector instruction (take-it-out timing).  The compiler does not know that these are MFMAs, so it puts
+// no wait states between one of them and a vector instruction that reads its result (an 8-pass MFMA needs 11).
+// The invariant that stands in for them: a score tile is first read two or more MFMAs (64 cycles) after the last
+// product into it.  It is kept in the source, not left to the scheduler - the statements are volatile (their order
+// among themselves and against the other pinned statements is the written one), inside a step every MFMA and the
+// softmax slices behind it sit between scheduling barriers, and where no MFMAs separate a tile's last product from
+// its first reader (the prologue) scores_settled() spends the wait states and ties the tile behind them.  The
+// accumulating form reads exactly the registers it writes, the one dependent sequence that the matrix pipe
+// forwards by itself.
 DFHIP_DEVICE f32x16 mfma_scores_first(bf16x8 k_rows, bf16x8 q_frag) {
   f32x16 d;
-  asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(k_rows), "a"(q_frag));
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(k_rows), "a"(q_frag));
   return d;
 }
 DFHIP_DEVICE void mfma_scores_next(f32x16& d, bf16x8 k_rows, bf16x8 q_frag) {
-  asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(k_rows), "a"(q_frag));
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(k_rows), "a"(q_frag));
+}
+// 12 wait states, and every later use of the two halves of a score tile tied behind them.
+DFHIP_DEVICE void scores_settled(f32x16 (&s)[2]) {
+  asm volatile("s_nop 7\n\ts_nop 3" : "+v"(s[0]), "+v"(s[1]));
+  DFHIP_PIN;
 }
 
 DFHIP_DEVICE int pi(int m) {   // MFMA row -> position inside a 32-position tile
@@ -243,6 +253,10 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
     }
   };
 
+  // Hazard invariant of a step (see mfma_scores_first): s_out's last products are the step's last two MFMAs (nb = 0,
+  // then nb = 1); the next step reads s_in[0] behind its second MFMA at the earliest and s_in[1] sixteen slices
+  // later, i.e. two or more MFMAs after the last product into the registers it reads, and the scheduling barrier
+  // behind every MFMA keeps it so.
   // One step: P V of tile [vb, vsb] (probabilities pf_in) with the two row-sum MFMAs of each k-step behind
   // it, then - DO_S - the scores of tile [kb, ksb] into s_out, with - DO_SM - the softmax of tile [mb, msb]
   // (scores s_in -> pf_out) sliced between the MFMAs.  A fragments are read AHEAD MFMA pairs ahead; the
@@ -334,6 +348,10 @@ causal_attention_kernel(const uint16_t* __restrict__ q, int64_t ld_q, const uint
       }
     }
   }
+  // nothing but the products into sB separates sA's last product from its first reader, and the scheduler is
+  // free to put those elsewhere: the wait states are spent here, for both tiles
+  scores_settled(sA);
+  scores_settled(sB);
   first_tile_reference(last_block_wave == 0, sA);
   if (last_block_wave == 0) {
 #pragma unroll

@@ -79,8 +79,9 @@ DFHIP_DEVICE float wave_max(float v) {
 // i % 8) and each XCD has a private L2.  remap_xcd turns the launch index into
 // a tile index such that every XCD walks one contiguous range of tiles, so the
 // tiles that are resident together on an XCD are neighbours and share operand
-// rows/columns in that XCD's L2.
-DFHIP_DEVICE int remap_xcd(int pid, int total) {
+// rows/columns in that XCD's L2.  (Also compiled for the host: the mapping is
+// replayed by CPU tests.)
+__host__ __device__ __forceinline__ int remap_xcd(int pid, int total) {
   constexpr int XCDS = 8;
   const int xcd = pid % XCDS;
   const int local = pid / XCDS;
@@ -88,6 +89,16 @@ DFHIP_DEVICE int remap_xcd(int pid, int total) {
   const int rem = total % XCDS;
   const int start = xcd * base + (xcd < rem ? xcd : rem);
   return start + local;
+}
+
+// Work item of a workgroup of the 256 x 256 split-K launch (`tiles` tiles, K of every tile cut into
+// `split_k` parts): the launch is part-major - launch indices [p * tiles, (p + 1) * tiles) are part p of
+// every tile, dealt to the XCDs like the tiles of an unsplit launch.  The last part of a tile, which waits
+// for the others, therefore has the highest launch index of that tile for every tile count, and the parts
+// it waits for were dispatched before it.
+__host__ __device__ __forceinline__ void splitk_work_of(int pid, int tiles, int& tile, int& part) {
+  part = pid / tiles;
+  tile = remap_xcd(pid - part * tiles, tiles);
 }
 
 // ---- hand-ordered memory operations of the LDS-DMA GEMM kernels ------------------------------

@@ -289,9 +289,8 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave & 1, wave_n = wave >> 1;
 
-  const int work = remap_xcd(blockIdx.x, tiles_m * tiles_n * split_k);
-  const int tile = work / split_k;
-  const int part = work - tile * split_k;
+  int tile, part;
+  splitk_work_of(blockIdx.x, tiles_m * tiles_n, tile, part);
   const int per_panel = GROUP_M * tiles_n;
   const int first_m = (tile / per_panel) * GROUP_M;
   const int rows_in_panel = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
@@ -415,9 +414,10 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   if (!FUSED && split_k > 1) {
     // Parts 0 .. split_k-2 of a tile leave their fp32 block in `partials`, count themselves in and are
     // done; the last part waits for that count, adds the blocks to its own accumulators in part order (so the
-    // sum has one order) and writes the tile.  The last part has the highest launch index of its tile and
-    // workgroups start in launch order, so whoever it waits for is already running or finished - and those
-    // never wait for anybody.  The wait is bounded; a tile whose parts never arrived is filled with NaN.
+    // sum has one order) and writes the tile.  The launch is part-major (splitk_work_of), so the last part has
+    // the highest launch index of its tile, and workgroups are dispatched in launch order: whoever it waits for
+    // is already running or finished - and those never wait for anybody.  The wait is bounded; a tile whose
+    // parts never arrived is filled with NaN.
     int* const counter = arrivals + tile;
     if (part != split_k - 1) {
       f32x4* mine = reinterpret_cast<f32x4*>(partials) + ((int64_t)tile * split_k + part) * (64 * RTHREADS) + tid;
@@ -1654,6 +1654,14 @@ extern "C" int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void*
                             static_cast<hipStream_t>(stream));
 }
 
+extern "C" int dfhip_gemm_bf16_splitk_work(int launch_index, int tiles, int split_k, int* tile, int* part) {
+  if (!tile || !part) return DFHIP_ERR_NULL_POINTER;
+  if (tiles < 1 || split_k < 1 || launch_index < 0 || (int64_t)launch_index >= (int64_t)tiles * split_k)
+    return DFHIP_ERR_BAD_ARGUMENT;
+  splitk_work_of(launch_index, tiles, *tile, *part);
+  return DFHIP_OK;
+}
+
 extern "C" int dfhip_gemm_bf16_gate_up_silu(const void* A, int64_t lda, const void* W_gate, const void* W_up,
                                             int64_t ldw, void* Out, int64_t ldo, int M, int I, int K,
                                             dfhip_stream_t stream) {
@@ -1723,12 +1731,15 @@ constexpr int MAX_DEVICES = 64;
 std::mutex scratch_mutex;
 void* scratch_ptr[MAX_DEVICES];   // device address of `scratch` on each GPU, looked up on first use
 
-// The address of this GPU's copy of `scratch` (null: the lookup failed).  No allocation happens here.
-void* scratch_on_current_device() {
+// The address of this GPU's copy of `scratch` (null: not known and not to be looked up now).  The lookup
+// (hipGetSymbolAddress, once per device) may set up the code object's device variables, which is not a thing to
+// do while a stream is capturing: with `may_look_up` false only an address found earlier is returned.  No
+// allocation happens here.
+void* scratch_on_current_device(bool may_look_up) {
   int device = -1;
   if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= MAX_DEVICES) return nullptr;
   std::lock_guard<std::mutex> guard(scratch_mutex);
-  if (!scratch_ptr[device]) {
+  if (!scratch_ptr[device] && may_look_up) {
     void* p = nullptr;
     if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) {
       (void)hipGetLastError();
@@ -1749,8 +1760,14 @@ extern "C" int dfhip_gemm_bf16_nt_splitk_static(const void* A, int64_t lda, cons
   if (need > (size_t)DFHIP_SPLITK_STATIC_BYTES) return DFHIP_ERR_TOO_LARGE;
   void* ws = nullptr;
   if (split_k > 1) {
-    ws = scratch_on_current_device();
-    if (!ws) return DFHIP_ERR_NO_DEVICE;
+    // the first call on a device finds the array's address and must not be part of a capture
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capturing) != hipSuccess) {
+      (void)hipGetLastError();
+      return DFHIP_ERR_LAUNCH;
+    }
+    ws = scratch_on_current_device(capturing == hipStreamCaptureStatusNone);
+    if (!ws) return capturing == hipStreamCaptureStatusNone ? DFHIP_ERR_NO_DEVICE : DFHIP_ERR_BAD_ARGUMENT;
     // The array keeps what the last call left.  Completed launches leave the counters at zero; they are
     // cleared all the same (a fill kernel, not a memset node), so that a launch that never finished cannot
     // poison the next one.  The two split-K kernels size their counter areas differently; the larger one is

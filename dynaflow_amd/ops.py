@@ -95,7 +95,11 @@ def _require_device(*tensors: torch.Tensor) -> None:
 #: nano-batch are chained one after the other whatever streams they run on; different nano-batches, and the
 #: forwards of different engines, may overlap and must not share arrival counters.  Outside: one per (device, stream).
 _splitk_workspaces: dict[tuple, torch.Tensor] = {}
-#: workspaces that were replaced by larger ones: captured graphs may still point at them
+#: addresses of workspaces that were handed to a launch while its stream was capturing: a graph may replay
+#: against them for as long as it lives
+_captured_workspaces: set[int] = set()
+#: workspaces that were replaced by larger ones and that a captured graph may still point at (one per capture
+#: at most: a replaced workspace that no capture ever saw is given back to the allocator)
 _retired_workspaces: list[torch.Tensor] = []
 #: split K for shapes with too few tiles (DYNAFLOW_SPLIT_K=0 switches it off)
 SPLIT_K_ENABLED = os.environ.get("DYNAFLOW_SPLIT_K", "1") != "0"
@@ -137,9 +141,12 @@ def _zeroed_workspace(cache: dict, device: torch.device, stream: int, nbytes: in
     else:
         key = (device.index or 0, "stream", stream)
     ws = cache.get(key)
+    capturing = torch.cuda.is_current_stream_capturing()
     if ws is not None and ws.numel() >= nbytes:
+        if capturing:
+            _captured_workspaces.add(ws.data_ptr())
         return ws
-    if torch.cuda.is_current_stream_capturing():
+    if capturing:
         # No buffer from an eager launch to fall back on: this one comes from the graph's memory pool and its
         # start is zeroed by a fill kernel that is part of the graph (a kernel, not a memset node).
         ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
@@ -147,7 +154,10 @@ def _zeroed_workspace(cache: dict, device: torch.device, stream: int, nbytes: in
         _cabi.check("dfhip_fill_u32", rc)
         return ws
     if ws is not None:
-        _retired_workspaces.append(ws)
+        if ws.data_ptr() in _captured_workspaces:
+            _retired_workspaces.append(ws)
+        else:
+            ws.record_stream(torch.cuda.current_stream())   # launches already queued on this stream still use it
     ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
     cache[key] = ws
     return ws
@@ -274,6 +284,8 @@ class StackedWeightCache:
         self.enabled = os.environ.get("DYNAFLOW_STACK_WEIGHTS", "1") != "0"
         self._entries: dict[tuple, torch.Tensor] = {}
         self._keys_of_member: dict[int, set] = {}       # id(member) -> keys of the entries it belongs to
+        # finalizers run on whatever thread drops the last reference to a weight
+        self._lock = threading.RLock()
 
     @staticmethod
     def key_of(weights) -> tuple:
@@ -283,44 +295,47 @@ class StackedWeightCache:
         return len(self._entries)
 
     def _drop_member(self, member_id: int) -> None:
-        for key in self._keys_of_member.pop(member_id, ()):
-            self._entries.pop(key, None)
+        with self._lock:
+            for key in self._keys_of_member.pop(member_id, ()):
+                self._entries.pop(key, None)
 
     def get(self, weights, build):
         """The concatenation for ``weights``; ``build()`` makes it when there is none (it may return None: no
         entry is kept then)."""
         key = self.key_of(weights)
-        stacked = self._entries.get(key)
-        if stacked is not None:
+        with self._lock:
+            stacked = self._entries.get(key)
+            if stacked is not None:
+                return stacked
+            stacked = build()
+            if stacked is None:
+                return None
+            for w in weights:
+                known = self._keys_of_member.get(id(w))
+                if known is None:
+                    known = self._keys_of_member[id(w)] = set()
+                    weakref.finalize(w, self._drop_member, id(w))
+                else:
+                    # the same tensor with another address or version: its older concatenations are stale
+                    for old in [k for k in known if k != key]:
+                        self._entries.pop(old, None)
+                        known.discard(old)
+                known.add(key)
+            self._entries[key] = stacked
             return stacked
-        stacked = build()
-        if stacked is None:
-            return None
-        for w in weights:
-            known = self._keys_of_member.get(id(w))
-            if known is None:
-                known = self._keys_of_member[id(w)] = set()
-                weakref.finalize(w, self._drop_member, id(w))
-            else:
-                # the same tensor with another address or version: its older concatenations are stale
-                for old in [k for k in known if k != key]:
-                    self._entries.pop(old, None)
-                    known.discard(old)
-            known.add(key)
-        self._entries[key] = stacked
-        return stacked
 
     def invalidate(self, weights=None) -> None:
         """Drop every entry (``weights`` None) or the entries that any of ``weights`` belongs to."""
-        if weights is None:
-            self._entries.clear()
-            for known in self._keys_of_member.values():
-                known.clear()
-            return
-        for w in weights:
-            for key in list(self._keys_of_member.get(id(w), ())):
-                self._entries.pop(key, None)
-                self._keys_of_member[id(w)].discard(key)
+        with self._lock:
+            if weights is None:
+                self._entries.clear()
+                for known in self._keys_of_member.values():
+                    known.clear()
+                return
+            for w in weights:
+                for key in list(self._keys_of_member.get(id(w), ())):
+                    self._entries.pop(key, None)
+                    self._keys_of_member[id(w)].discard(key)
 
 
 _stacked_weights = StackedWeightCache()

@@ -116,10 +116,12 @@ int dfhip_gemm_bf16_plan_shared(int M, int N, int K, int share, int* variant, in
  * projections examples/ae/scheduler/hf/nanoflow.py:30 names: [2048,14336] x [4096,14336]^T has 128 tiles of 256x256 for 256
  * compute units).  Each tile is computed by `split_k` workgroups over disjoint
  * K ranges.  With the 256x256 ring kernel parts 0 .. split_k-2 leave their fp32
- * block in `workspace` and count themselves in; the last part - the one with the
- * highest launch index of its tile, so whoever it waits for was started before
- * it - waits for that count, adds the blocks to its own sum in part order
- * (deterministic) and writes C.  The wait is bounded (about a second); a tile
+ * block in `workspace` and count themselves in; the last part waits for that
+ * count, adds the blocks to its own sum in part order (deterministic) and writes
+ * C.  The launch is part-major (workgroups [p * tiles, (p + 1) * tiles) are part
+ * p of every tile, see dfhip_gemm_bf16_splitk_work), so the part that waits has
+ * the highest launch index of its tile for every tile count and whoever it waits
+ * for was dispatched before it.  The wait is bounded (about a second); a tile
  * whose parts never arrived is written as NaN.  With the weight-streaming kernel
  * (variant 6) every part leaves a block and the part that arrives last adds them
  * up; nobody waits.  `workspace` (device memory, 16-byte aligned,
@@ -132,6 +134,12 @@ size_t dfhip_gemm_bf16_splitk_workspace_bytes(int M, int N, int split_k);
 int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                               int64_t ldc, int M, int N, int K, int split_k, void* workspace,
                               size_t workspace_bytes, dfhip_stream_t stream);
+/* Host-side replay of the launch order of the 256x256 split-K kernel: which tile and which part of K
+ * the workgroup with launch index `launch_index` computes in a launch over `tiles` tiles (launch
+ * indices 0 .. tiles * split_k - 1).  Touches no device; it exists so that the ordering argument above
+ * (the waiting part is the last of its tile to be dispatched) can be checked on any machine.  No
+ * counterpart in the reference. */
+int dfhip_gemm_bf16_splitk_work(int launch_index, int tiles, int split_k, int* tile, int* part);
 
 /* dfhip_gemm_bf16_nt_splitk without a workspace argument and without any allocation: the arrival
  * counters and fp32 partial blocks live in a device array of DFHIP_SPLITK_STATIC_BYTES that is part
@@ -144,7 +152,11 @@ int dfhip_gemm_bf16_nt_splitk(const void* A, int64_t lda, const void* W, int64_t
  * [2048,14336] x [4096,14336]^T with split_k = 2).  All calls on one GPU share the one array: calls
  * that may overlap in time on a GPU (different streams, different threads) race and must use
  * dfhip_gemm_bf16_nt_splitk with workspaces of their own.  The counters are cleared by a small fill
- * kernel ahead of the GEMM on `stream` (no memset node), so the call is legal under capture. */
+ * kernel ahead of the GEMM on `stream` (no memset node), so the call is legal under capture - once
+ * the library knows where the array lives on that GPU: the first call with split_k > 1 on a device
+ * looks the address up and must be made on a stream that is not capturing (under capture before
+ * that it is refused with DFHIP_ERR_BAD_ARGUMENT and launches nothing).  The kernel is the one
+ * dfhip_gemm_bf16_nt_splitk picks for the shape (its plan for a lone launch) with the caller's split_k. */
 #define DFHIP_SPLITK_STATIC_BYTES ((64u << 20) + 4096u)
 int dfhip_gemm_bf16_nt_splitk_static(const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
                                      int64_t ldc, int M, int N, int K, int split_k,

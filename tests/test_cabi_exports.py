@@ -68,6 +68,64 @@ def test_argument_checks_run_before_any_launch():
     assert b"scratch" in lib.dfhip_status_string(-8)
 
 
+def _splitk_launch_order(lib, tiles, split_k):
+    """{tile: [(launch index, part), ...]} of a split-K launch, replayed on the host."""
+    tile, part = ctypes.c_int(-1), ctypes.c_int(-1)
+    order = {}
+    for pid in range(tiles * split_k):
+        assert lib.dfhip_gemm_bf16_splitk_work(pid, tiles, split_k, ctypes.byref(tile), ctypes.byref(part)) == 0
+        order.setdefault(tile.value, []).append((pid, part.value))
+    return order
+
+
+@pytest.mark.parametrize("tiles,split_k", [
+    (128, 2),            # down projection of a 2048-token nano-batch: [2048,14336] x [4096,14336]^T
+    (100, 2), (36, 7), (50, 5), (6, 3),     # tile counts that are no multiple of the 8 XCDs
+    (1, 8), (7, 8), (8, 8), (9, 2), (33, 4), (64, 4), (127, 2),
+])
+def test_split_k_waiter_is_the_last_of_its_tile_to_be_dispatched(tiles, split_k):
+    """The part of a tile that waits for the others (part split_k - 1) must have the highest launch index of that
+    tile: workgroups are dispatched in launch order, so everything it waits for is then running or done, whatever
+    the tile count and however few compute units the launch gets.  Also: every (tile, part) is computed exactly
+    once, and the parts of one K range are dealt to the XCDs (launch index % 8) in contiguous tile ranges."""
+    lib = _cabi.load()
+    order = _splitk_launch_order(lib, tiles, split_k)
+    assert sorted(order) == list(range(tiles))
+    for tile, work in order.items():
+        assert sorted(part for _, part in work) == list(range(split_k)), (tile, work)
+        waiter = max(work)                       # highest launch index of the tile
+        assert waiter[1] == split_k - 1, (tile, work)
+    for p in range(split_k):
+        by_xcd = {}
+        for tile, work in order.items():
+            pid = next(pid for pid, part in work if part == p)
+            by_xcd.setdefault(pid % 8, []).append(tile)
+        for tiles_of_xcd in by_xcd.values():
+            tiles_of_xcd.sort()
+            assert tiles_of_xcd == list(range(tiles_of_xcd[0], tiles_of_xcd[0] + len(tiles_of_xcd)))
+
+
+def test_split_k_planned_shapes_keep_the_waiter_last():
+    """The same for the split the plan picks on the shapes the layers use (and their side-by-side plans)."""
+    lib = _cabi.load()
+    variant, split_k = ctypes.c_int(0), ctypes.c_int(1)
+    seen = 0
+    for M in (256, 300, 512, 768, 1024, 1536, 2048, 4096, 8192):
+        for N, K in ((4096, 14336), (4096, 4096), (6144, 4096), (14336, 4096), (8192, 28672), (264, 512)):
+            for share in (1, 2, 4):
+                assert lib.dfhip_gemm_bf16_plan_shared(M, N, K, share, ctypes.byref(variant), ctypes.byref(split_k)) == 0
+                if variant.value != 0 or split_k.value < 2:
+                    continue
+                seen += 1
+                tiles = ((M + 255) // 256) * ((N + 255) // 256)
+                for tile, work in _splitk_launch_order(lib, tiles, split_k.value).items():
+                    assert max(work)[1] == split_k.value - 1, (M, N, K, share, tile, work)
+    assert seen > 0
+    bad = ctypes.c_int(0)
+    assert lib.dfhip_gemm_bf16_splitk_work(16, 8, 2, ctypes.byref(bad), ctypes.byref(bad)) == -7
+    assert lib.dfhip_gemm_bf16_splitk_work(0, 8, 2, None, ctypes.byref(bad)) == -1
+
+
 def test_operators_refuse_host_tensors():
     from dynaflow_amd import ops
 

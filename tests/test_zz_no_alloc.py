@@ -73,3 +73,39 @@ def test_static_scratch_split_k_refuses_what_does_not_fit():
                                                 stream) == 0
     torch.cuda.synchronize()
     assert float(c.float().abs().max()) == 0.0
+
+
+def test_static_scratch_split_k_under_graph_capture_replays_with_the_same_bits():
+    """Once the library knows the array's address on this GPU (any earlier call outside capture: here the eager
+    one) the call is legal in a captured graph: the counters are cleared by a fill kernel, no memset node and no
+    allocation are recorded.  Replayed three times with eager work and synchronisations in between; every replay
+    must give the bits of the eager call, also after the input changed."""
+    from dynaflow_amd import _cabi
+
+    lib = _cabi.load()
+    M, N, K, split_k = 768, 1024, 2048, 4
+    a = randn((M, K), 81).bfloat16().cuda()
+    w = randn((N, K), 82, 0.03).bfloat16().cuda()
+    eager = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    replayed = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+
+    def call(out):
+        rc = lib.dfhip_gemm_bf16_nt_splitk_static(a.data_ptr(), K, w.data_ptr(), K, out.data_ptr(), N, M, N, K,
+                                                  split_k, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+
+    print(f"split-K static under capture: M={M} N={N} K={K} split_k={split_k}", flush=True)
+    call(eager)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(replayed)
+    for round_ in range(3):
+        if round_:
+            a.copy_(randn((M, K), 83 + round_).bfloat16())     # eager work between the replays
+            call(eager)
+        replayed.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(eager, replayed), round_
