@@ -41,6 +41,7 @@ GATE_GEMM_TRAFFIC_BYTES = 432.9e6      # fetch 369.4 MB + write 63.5 MB
 GATE_UP_SILU_TRAFFIC_BYTES = 845.8e6   # fetch 738.9 MB + write 106.9 MB (non-temporal stores leave in 64-byte pieces:
                                        # runs that straddle two are counted twice; 58.7 MB of results)
 GATE_UP_SILU_SQUARE_TRAFFIC_BYTES = 797.3e6   # the 256 x (128 + 128) tile: fetch 738.6 MB + write 58.7 MB
+GATE_UP_SILU_PAIR_KERNEL = "gemm_bf16_ring_kernel<true>, 256 x (128 + 128) tile"
 METRIC = "MLP-layer tokens/s + overlap speedup vs serial, 8B-shape bf16, 1 MI355X"
 
 
@@ -52,6 +53,11 @@ def parse_args():
     p.add_argument("--skip-cpu", action="store_true", help="leave out the host baseline (profiling runs)")
     p.add_argument("--sustain-seconds", type=float, default=3.0,
                    help="seconds of continuous load ahead of the `sustained` figures (0: leave them out)")
+    p.add_argument("--settle-seconds", type=float, default=0.5,
+                   help="seconds of the same step, untimed, ahead of the warm-up steps of every timed loop (the "
+                        "package's clocks in their loaded state; 0: none)")
+    p.add_argument("--headline-config-only", action="store_true",
+                   help="leave out the `other_configs` object (decoder layer, fp8 layer, decode step)")
     p.add_argument("--kernels-only", action="store_true",
                    help="run only the single-kernel timing loops plus a 256 MiB device copy (used to calibrate "
                         "FETCH_SIZE / WRITE_SIZE under rocprofv3 --pmc); prints the kernel figures as JSON")
@@ -118,12 +124,22 @@ def build_path(torch, x, weights, **knobs):
     return manager, compiled
 
 
-def time_steps(torch, manager, compiled, x, steps, warmup, use_graph):
+def time_steps(torch, manager, compiled, x, steps, warmup, use_graph, settle_s=0.0):
+    """ms per step over exactly ``steps`` steps after ``warmup`` untimed ones, a device synchronisation on both
+    sides; ``settle_s`` seconds of the same step run before the warm-up steps (untimed)."""
     def step():
         manager.prepare(TOKENS, [TOKENS], use_cudagraph=use_graph)
         return compiled(x)
 
     with torch.no_grad():
+        if settle_s > 0:
+            step()                                   # set-up of the first call (graph capture) is not load
+            torch.cuda.synchronize()
+            until = time.perf_counter() + settle_s
+            while time.perf_counter() < until:
+                for _ in range(10):
+                    step()
+                torch.cuda.synchronize()
         for _ in range(warmup):
             y = step()
         torch.cuda.synchronize()
@@ -387,9 +403,15 @@ def prefill_attention_kernels(torch, ops, iters):
     }
 
 
-def fp8_config(torch, steps, warmup):
+def rel_err_of(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+
+
+def fp8_config(torch, steps, warmup, brief=False):
     """fp8 70B-shaped layer: x[8192,8192] bf16 quantised per tensor inside the graph, weights e4m3 with
-    per-output-channel scales, 4 nano-batches of 2048 through the manager on two streams."""
+    per-output-channel scales, 4 nano-batches of 2048 through the manager on two streams.  ``brief``: only the
+    reported mode and its one-stream baseline."""
     from dynaflow_amd.backend import make_backend
     from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
     from dynaflow_amd.fp8_mlp import Fp8SwiGLU
@@ -405,10 +427,15 @@ def fp8_config(torch, steps, warmup):
     layer = Fp8SwiGLU.from_weights(*parts)
     del parts
     results = {}
-    for name, knobs in (("serialized", {"serialize": True}), ("overlapped", {"whole_graph": True}),
-                        ("overlapped_fused_gate_up", {"whole_graph": True, "fuse_silu_epilogue": True}),
-                        ("stream_per_nano_batch_fused_gate_up", {"whole_graph": True, "fuse_silu_epilogue": True,
-                                                                 "streams": "by_nano_batch"})):
+    fused = {"whole_graph": True, "fuse_silu_epilogue": True}
+    modes = [("serialized", {"serialize": True}), ("overlapped", {"whole_graph": True}),
+             ("serialized_fused_gate_up", {"serialize": True, **fused}),
+             ("overlapped_fused_gate_up", dict(fused)),
+             ("stream_per_nano_batch_fused_gate_up", {**fused, "streams": "by_nano_batch"})]
+    if brief:
+        modes = [m for m in modes if m[0] in ("serialized_fused_gate_up", "overlapped_fused_gate_up")]
+    y_best = None
+    for name, knobs in modes:
         # the fused mode: gate, up and SiLU*mul + absmax in ONE GEMM launch, cut in front of the down projection
         layer.fuse_gate_up = bool(knobs.get("fuse_silu_epilogue", False))
         extra = {"min_nano_split_tokens": 64, "num_nano_batches": splits, "dump_graph": False, **EXTRA_KNOBS}
@@ -427,19 +454,23 @@ def fp8_config(torch, steps, warmup):
                 manager.prepare(tokens, [tokens], use_cudagraph=use_graph)
                 return compiled(x)
 
-            modes = (("eager", False),) if name == "serialized" else (("eager", False), ("graph", True))
-            for mode, use_graph in modes:
+            timed = (("eager", False),) if name == "serialized" else \
+                    (("graph", True),) if brief else (("eager", False), ("graph", True))
+            for mode, use_graph in timed:
                 for _ in range(warmup):
                     step(use_graph)
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
                 for _ in range(steps):
-                    step(use_graph)
+                    y = step(use_graph)
                 torch.cuda.synchronize()
                 results[f"{name}_{mode}_ms"] = (time.perf_counter() - t0) * 1e3 / steps
+            if name == "overlapped_fused_gate_up":
+                y_best = y.clone()
     flops = 6.0 * tokens * hidden * inter
-    best_mode = min(("overlapped_graph_ms", "overlapped_fused_gate_up_graph_ms",
-                     "stream_per_nano_batch_fused_gate_up_graph_ms"), key=lambda m: results[m])
+    candidates = [m for m in ("overlapped_graph_ms", "overlapped_fused_gate_up_graph_ms",
+                              "stream_per_nano_batch_fused_gate_up_graph_ms") if m in results]
+    best_mode = min(candidates, key=lambda m: results[m])
     best = results[best_mode]
     # the dominant kernel, alone: gate + up + SiLU*mul + absmax of one nano-batch in one launch
     from dynaflow_amd import _cabi, ops
@@ -458,15 +489,50 @@ def fp8_config(torch, steps, warmup):
 
     ms_fused = time_kernel(torch, fused_launch, 30)
     fused_flops = 4.0 * mb * hidden * inter
-    return {
+    del act, xq
+
+    # sampled rows of the fused mode's result against an evaluation that takes nothing from the kernels: torch's own
+    # e4m3 conversion of the activations, gate / up of the whole nano-batch as fp32 products of the dequantised
+    # operands (torch on the GPU), and - in the CPU leg - the oracle's SiLU*mul, its absmax over the whole
+    # nano-batch, the oracle's e4m3 encoder for the sampled rows, an fp32 down projection
+    prepared = []
+    if y_best is not None:
+        fp8_max = 448.0
+        with torch.no_grad():
+            wg = layer.w_gate_q.float() * layer.w_gate_s[:, None]
+            wu = layer.w_up_q.float() * layer.w_up_s[:, None]
+            for nano_batch, picked in ((0, [0, 777, 2047]), (3, [1, 2046])):
+                xb = x[nano_batch * mb:(nano_batch + 1) * mb].float()
+                x_scale = xb.abs().max().clamp_min(1e-12) / fp8_max
+                xd = (xb / x_scale).clamp(-fp8_max, fp8_max).to(torch.float8_e4m3fn).float() * x_scale
+                rows = torch.tensor(picked, device="cuda")
+                prepared.append(((xd @ wg.t()).bfloat16(), (xd @ wu.t()).bfloat16(), rows,
+                                 y_best[nano_batch * mb + rows].float()))
+            del wg, wu, xb, xd
+
+    def oracle_check(mods):
+        oracle_mlp = mods["mlp"]
+        errs = []
+        wd = layer.w_down_q.float() * layer.w_down_s[:, None]
+        for g, u, rows, got in prepared:
+            a = oracle_mlp.silu_mul_exact(g, u)
+            a_scale = a.float().abs().max().clamp_min(1e-12) / 448.0
+            scaled = (a[rows].float() / a_scale).clamp(-448.0, 448.0).cpu()
+            codes = torch.from_numpy(oracle_mlp.e4m3_encode(scaled.numpy()))
+            a_rows = oracle_mlp.dequant(codes, a_scale.reshape(1).cpu())
+            errs.append(rel_err_of(got, a_rows.cuda() @ wd.t()))
+        return {"worst": max(errs), "bound": 5e-2, "rows": "3 of nano-batch 0, 2 of nano-batch 3",
+                "against": "fp32 evaluation of the dequantised operands, re-quantisation by the oracle's encoder"}
+
+    line = {
         "metric": "fp8 MLP-layer tokens/s, 70B-shape e4m3, 1 MI355X",
         "value": tokens / (best * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": best, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3",
         "data": "synthetic",
         "config": {"workload": "fp8 70B-shaped SwiGLU MLP layer, x[8192,8192], I=28672, 4 nano-batches of 2048, "
-                               "per-tensor activation / per-channel weight scales, bf16 output; the best of "
-                               "the separate gate / up / SiLU*mul launches and the one-launch form (streams by "
-                               "sub-graph kind or one per nano-batch) is reported",
+                               "per-tensor activation / per-channel weight scales, bf16 output; gate / up / "
+                               "SiLU*mul + absmax as one launch per nano-batch, then re-quantisation and the down "
+                               "projection; whole two-stream schedule as one hipGraph",
                    "issue_mode": best_mode[:-3]},
         "timings": results,
         "layer": {"tflops": flops / (best * 1e-3) / 1e12, "frac_of_fp8_mfma_peak": flops / (best * 1e-3) / 1e12 / 5000.0},
@@ -479,11 +545,17 @@ def fp8_config(torch, steps, warmup):
             # written; the summary is under profiles/); algorithmic: 16.8 + 2 x 234.9 MB read, 117.4 MB written
             "traffic": 1527.9e6, "traffic_unit": "bytes per launch",
         },
-        "overlap_speedup": results["serialized_eager_ms"] / best,
+        "oracle_check": oracle_check if prepared else None,
     }
+    if "serialized_fused_gate_up_graph_ms" in results and "overlapped_fused_gate_up_graph_ms" in results:
+        # the same kernels and split on one stream against the two-stream schedule, graph against graph
+        line["overlap_speedup"] = results["serialized_fused_gate_up_graph_ms"] / results["overlapped_fused_gate_up_graph_ms"]
+    if "serialized_eager_ms" in results:
+        line["speedup_vs_separate_kernels_serialized_eager"] = results["serialized_eager_ms"] / best
+    return line
 
 
-def decoder_config(torch, steps, warmup):
+def decoder_config(torch, steps, warmup, brief=False):
     """Full decoder layer, random-init bf16: hidden 4096, 32 q / 8 kv heads, head_dim 128, RoPE theta 5e5,
     causal attention, SwiGLU 14336; prefill batch 8 x seq 2048, tokens ~ U[0, 128256)."""
     from dynaflow_amd.backend import make_backend
@@ -504,11 +576,19 @@ def decoder_config(torch, steps, warmup):
     ids = torch.randint(0, vocab, (batch * S,), generator=torch.Generator().manual_seed(4)).cuda()
     T = batch * S
     results = {}
-    for name, knobs in (("serialized", {"serialize": True}), ("overlapped", {"whole_graph": True}),
-                        ("overlapped_fused_silu", {"whole_graph": True, "fuse_silu_epilogue": True}),
-                        # every nano-batch on a stream of its own instead of one stream per kind of sub-graph
-                        ("stream_per_nano_batch_fused_silu", {"whole_graph": True, "fuse_silu_epilogue": True,
-                                                              "streams": "by_nano_batch"})):
+    modes = [("serialized", {"serialize": True}), ("overlapped", {"whole_graph": True}),
+             ("overlapped_fused_silu", {"whole_graph": True, "fuse_silu_epilogue": True}),
+             # every nano-batch on a stream of its own instead of one stream per kind of sub-graph (kernels planned
+             # for the two launches of a kind that then run side by side)
+             ("stream_per_nano_batch_fused_silu", {"whole_graph": True, "fuse_silu_epilogue": True,
+                                                   "streams": "by_nano_batch"}),
+             # the same kernels and split as the mode above on ONE stream: the baseline of the overlap figure
+             ("one_stream_same_kernels", {"whole_graph": True, "fuse_silu_epilogue": True, "serialize": True,
+                                          "side_by_side": 2})]
+    if brief:
+        modes = modes[3:]
+    y_best = None
+    for name, knobs in modes:
         extra = {"min_nano_split_tokens": 64, "dump_graph": False, **EXTRA_KNOBS}
         extra.update(knobs)
         cfg = DynaFlowConfig("dynaflow_amd.schedulers:DecoderOverlapScheduler", 2, InductorConfig(enabled=True),
@@ -520,8 +600,9 @@ def decoder_config(torch, steps, warmup):
         with torch.no_grad():
             manager.prepare(batch, [S] * batch)
             compiled(ids)
-            modes = (("eager", False),) if name == "serialized" else (("eager", False), ("graph", True))
-            for mode, use_graph in modes:
+            timed = (("eager", False),) if name == "serialized" else \
+                    (("graph", True),) if brief or name == "one_stream_same_kernels" else (("eager", False), ("graph", True))
+            for mode, use_graph in timed:
                 for _ in range(warmup):
                     manager.prepare(batch, [S] * batch, use_cudagraph=use_graph)
                     compiled(ids)
@@ -529,12 +610,14 @@ def decoder_config(torch, steps, warmup):
                 t0 = time.perf_counter()
                 for _ in range(steps):
                     manager.prepare(batch, [S] * batch, use_cudagraph=use_graph)
-                    compiled(ids)
+                    y = compiled(ids)
                 torch.cuda.synchronize()
                 results[f"{name}_{mode}_ms"] = (time.perf_counter() - t0) * 1e3 / steps
+            if name == "stream_per_nano_batch_fused_silu":
+                y_best = y.clone()
     flops = 2.0 * T * H * 6144 + 2.0 * T * H * H + 2.0 * batch * 32 * S * S * 128 + 6.0 * T * H * I
-    candidates = ("overlapped_graph_ms", "overlapped_eager_ms", "overlapped_fused_silu_graph_ms",
-                  "stream_per_nano_batch_fused_silu_graph_ms")
+    candidates = [m for m in ("overlapped_graph_ms", "overlapped_eager_ms", "overlapped_fused_silu_graph_ms",
+                              "stream_per_nano_batch_fused_silu_graph_ms") if m in results]
     best_mode = min(candidates, key=lambda m: results[m])
     best = results[best_mode]
     # the dominant kernel, alone: gate + up + SiLU*mul of one nano-batch (8192 tokens) in one launch
@@ -546,7 +629,17 @@ def decoder_config(torch, steps, warmup):
     with torch.no_grad():
         ms_fused = time_kernel(torch, lambda: ops.gate_up_silu(xb, w_gate, w_up), 20)
     fused_flops = 4.0 * mb * H * I
-    return {
+    ids_host = ids.cpu()
+    rows = [255, 2047, 5 * S + 1000]             # two sequences, one of each nano-batch
+    got_rows = y_best[rows].float().cpu() if y_best is not None else None
+
+    def oracle_check(mods):
+        ref = mods["decoder"]
+        want = ref.decoder_layer_rows(ids_host, ref.params_of(layer), rows, S, 32, 8, 128)
+        return {"worst": rel_err_of(got_rows, want), "bound": 2e-2, "rows": rows,
+                "against": "float64 oracle of the layer restricted to the sampled rows' sequences"}
+
+    line = {
         "metric": "decoder-layer prefill tokens/s, 8B-shape bf16, 1 MI355X",
         "value": T / (best * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": best, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
@@ -568,11 +661,18 @@ def decoder_config(torch, steps, warmup):
             # written; the summary is under profiles/); algorithmic: 67.1 + 2 x 117.4 MB read, 234.9 MB written
             "traffic": 3056.8e6, "traffic_unit": "bytes per launch",
         },
-        "overlap_speedup": results["serialized_eager_ms"] / best,
+        "oracle_check": oracle_check if got_rows is not None else None,
     }
+    if "one_stream_same_kernels_graph_ms" in results and "stream_per_nano_batch_fused_silu_graph_ms" in results:
+        # the same kernels and split on one stream against the two-stream schedule, graph against graph
+        line["overlap_speedup"] = (results["one_stream_same_kernels_graph_ms"]
+                                   / results["stream_per_nano_batch_fused_silu_graph_ms"])
+    if "serialized_eager_ms" in results:
+        line["speedup_vs_separate_kernels_serialized_eager"] = results["serialized_eager_ms"] / best
+    return line
 
 
-def decode_config(torch, steps, warmup, layers=32):
+def decode_config(torch, steps, warmup, layers=32, brief=False):
     """Decode step: 256 sequences, one new token each, KV caches of 2048 positions ~N(0,1), 2 nano-batches of
     128; attention sub-graph of one nano-batch beside the MLP sub-graph of the other in every layer."""
     from dynaflow_amd.backend import make_backend
@@ -595,21 +695,31 @@ def decode_config(torch, steps, warmup, layers=32):
     # the last mode is the comparison without nano-batches: all 256 queries as one batch on one stream (the
     # weights are read once per step instead of once per nano-batch, nothing overlaps), sub-graphs replayed
     # "whole" modes: the complete two-stream schedule of all layers captured once and replayed as ONE hipGraph
-    for name, knobs, graphs in (("serialized_eager", {"serialize": True}, False), ("overlapped_eager", {}, False),
-                                ("overlapped_sub_graph_replay", {}, True),
-                                ("stream_per_nano_batch_sub_graph_replay", {"streams": "by_nano_batch"}, True),
-                                ("serialized_whole_graph", {"serialize": True, "whole_graph": True}, "whole"),
-                                ("overlapped_whole_graph", {"whole_graph": True}, "whole"),
-                                ("stream_per_nano_batch_whole_graph",
-                                 {"streams": "by_nano_batch", "whole_graph": True}, "whole"),
-                                # the same two modes with the kernels planned for two launches that share the GPU
-                                # (knob side_by_side: the weight-streaming GEMMs split K over half as many
-                                # workgroups and move half as many fp32 blocks; another order of additions)
-                                ("stream_per_nano_batch_planned_for_two_sub_graph_replay",
-                                 {"streams": "by_nano_batch", "side_by_side": 2}, True),
-                                ("stream_per_nano_batch_planned_for_two_whole_graph",
-                                 {"streams": "by_nano_batch", "side_by_side": 2, "whole_graph": True}, "whole"),
-                                ("unsplit_sub_graph_replay", {"min_nano_split_tokens": 1 << 30}, True)):
+    modes = [("serialized_eager", {"serialize": True}, False), ("overlapped_eager", {}, False),
+             ("overlapped_sub_graph_replay", {}, True),
+             # one stream per nano-batch with the kernels planned as lone launches (override of what the
+             # manager derives from the stream policy), for comparison
+             ("stream_per_nano_batch_planned_alone_sub_graph_replay",
+              {"streams": "by_nano_batch", "side_by_side": 1}, True),
+             ("serialized_whole_graph", {"serialize": True, "whole_graph": True}, "whole"),
+             ("overlapped_whole_graph", {"whole_graph": True}, "whole"),
+             ("stream_per_nano_batch_planned_alone_whole_graph",
+              {"streams": "by_nano_batch", "side_by_side": 1, "whole_graph": True}, "whole"),
+             # one stream per nano-batch: the same sub-graph of both nano-batches runs at the same time and
+             # the kernels are planned for the pair (the weight-streaming GEMMs split K over half as many
+             # workgroups and move half as many fp32 blocks; another order of additions)
+             ("stream_per_nano_batch_planned_for_two_sub_graph_replay", {"streams": "by_nano_batch"}, True),
+             ("stream_per_nano_batch_planned_for_two_whole_graph",
+              {"streams": "by_nano_batch", "whole_graph": True}, "whole"),
+             # the same kernels and split as the mode above on ONE stream: the baseline of the overlap figure
+             ("one_stream_same_kernels_whole_graph",
+              {"serialize": True, "side_by_side": 2, "whole_graph": True}, "whole"),
+             ("unsplit_sub_graph_replay", {"min_nano_split_tokens": 1 << 30}, True)]
+    if brief:
+        modes = [m for m in modes if m[0] in ("stream_per_nano_batch_planned_for_two_whole_graph",
+                                              "one_stream_same_kernels_whole_graph")]
+    y_best = None
+    for name, knobs, graphs in modes:
         extra = {"min_nano_split_tokens": 1, "dump_graph": False, "max_tokens": seqs, "fuse_silu_epilogue": True,
                  **EXTRA_KNOBS}
         extra.update(knobs)
@@ -636,31 +746,78 @@ def decode_config(torch, steps, warmup, layers=32):
             t0 = time.perf_counter()
             for _ in range(steps):
                 manager.prepare(seqs, [1] * seqs, use_cudagraph=bool(graphs))
-                compiled(*inputs)
+                y = compiled(*inputs)
             torch.cuda.synchronize()
             results[f"{name}_ms"] = (time.perf_counter() - t0) * 1e3 / steps
             if graphs == "whole":
                 assert len(manager._schedule_graphs) == 1, "the step was not replayed as one graph"
+            if name == "stream_per_nano_batch_planned_for_two_whole_graph":
+                y_best = y.clone()
         del manager, compiled
     weight_bytes = layers * 2.0 * ((heads + 2 * kv_heads) * 128 * H + H * heads * 128 + 3 * H * I)
     kv_bytes = layers * 2.0 * seqs * kv_heads * capacity * 128 * 2
     # reported beside the two-stream nano-batch modes, never as `value`: the unsplit batch, and the serialized
     # issue of the same nano-batches (the baseline of the overlap figure)
     aside = {k: results.pop(k) for k in ("unsplit_sub_graph_replay_ms", "serialized_eager_ms",
-                                          "serialized_whole_graph_ms")}
+                                          "serialized_whole_graph_ms", "one_stream_same_kernels_whole_graph_ms")
+             if k in results}
     best_mode = min(results, key=results.get)
     best = results[best_mode]
     results.update(aside)
-    return {
+
+    sampled = [0, 127, 255]
+    got_rows = y_best[sampled].float().cpu() if y_best is not None else None
+
+    def oracle_check(mods):
+        """The float64 oracle on the sampled tokens (a token's result depends on its own sequence only).  A decode
+        step with fixed lengths rewrites only the position it appends to, which the oracle writes too, so the
+        caches can be read after the timed steps."""
+        from dynaflow_amd.decode import unpack_v_cache
+
+        ref = mods["decode"]
+        rows = slots[sampled].long()
+
+        class Params(dict):
+            def __getitem__(self, name):
+                if name == "embed":
+                    return model.embed.detach()[ids[sampled]].double().cpu()
+                kind, i = name.rsplit(".", 1)
+                a, m = model.attn[int(i)], model.mlp[int(i)]
+                t = {"attn_norm": a.norm_weight, "wqkv": a.wqkv, "wo": a.wo, "mlp_norm": m.norm_weight,
+                     "w_gate": m.w_gate, "w_up": m.w_up, "w_down": m.w_down}[kind]
+                return t.detach().double().cpu()
+
+        class Caches:
+            def __init__(self, values):
+                self.values = values
+
+            def __len__(self):
+                return layers
+
+            def __getitem__(self, i):
+                a = model.attn[i]
+                c = unpack_v_cache(a.v_cache[rows]) if self.values else a.k_cache[rows]
+                return c.double().cpu().permute(0, 2, 1, 3).contiguous()
+
+        local = torch.arange(len(sampled))
+        want = ref.decode_step(local, local, lengths[sampled].cpu(), Params(), Caches(False), Caches(True), heads,
+                               kv_heads)
+        return {"worst": rel_err_of(got_rows, want), "bound": 0.1, "rows": sampled,
+                "against": "float64 oracle over all 32 layers on the sampled tokens; the bf16 roundings of the "
+                           "residual stream add up over the layers (eager PyTorch in bf16 is 0.04 from the same "
+                           "oracle), one layer's arithmetic is held to 2e-2 by the test suite"}
+
+    line = {
         "metric": "decode-step tokens/s, 32 x 8B-shaped layers, bf16, 1 MI355X",
         "value": seqs / (best * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": best, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"decode step over {layers} Llama-3-8B-shaped layers, {seqs} single-token queries, "
-                               f"{capacity} cached positions per sequence, 2 nano-batches of {half}; the best of "
-                               "the eager two-stream schedule, per-sub-graph graph replay and the whole split "
-                               "schedule replayed as one hipGraph (streams by sub-graph kind or one per "
-                               "nano-batch) is reported",
+                               f"{capacity} cached positions per sequence, 2 nano-batches of {half}, attention "
+                               "sub-graph and MLP sub-graph per layer; the fastest of the issue modes timed in "
+                               "this run is reported and named in issue_mode (by default: one stream per "
+                               "nano-batch, kernels planned for the two launches of a kind that run side by side, "
+                               "the whole split schedule replayed as one hipGraph)",
                    "issue_mode": best_mode[:-3]},
         "timings": results,
         "roofline": {"bound": "hbm", "achieved": (weight_bytes + kv_bytes) / (best * 1e-3) / 1e9,
@@ -668,8 +825,17 @@ def decode_config(torch, steps, warmup, layers=32):
                      "frac": (weight_bytes + kv_bytes) / (best * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "algorithmic_bytes": weight_bytes + kv_bytes,
                      "note": "weights counted once per step (each nano-batch reads them again: 2x in practice)"},
-        "overlap_speedup": min(results["serialized_eager_ms"], results["serialized_whole_graph_ms"]) / best,
+        "oracle_check": oracle_check if got_rows is not None else None,
     }
+    if "one_stream_same_kernels_whole_graph_ms" in results and \
+            "stream_per_nano_batch_planned_for_two_whole_graph_ms" in results:
+        # the same kernels and split on one stream against the two-stream schedule, graph against graph
+        line["overlap_speedup"] = (results["one_stream_same_kernels_whole_graph_ms"]
+                                   / results["stream_per_nano_batch_planned_for_two_whole_graph_ms"])
+    if "serialized_eager_ms" in results:
+        line["speedup_vs_serialized_lone_plans"] = min(results["serialized_eager_ms"],
+                                                       results["serialized_whole_graph_ms"]) / best
+    return line
 
 
 def synthetic_inputs(torch, tokens, hidden, inter, dtype):
@@ -686,12 +852,20 @@ def synthetic_inputs(torch, tokens, hidden, inter, dtype):
             normal(3, (hidden, inter), 0.02).to(dtype))
 
 
-def cpu_baseline(torch, sampled=None):
+def cpu_baseline(torch, sampled=None, other_checks=None, time_it=True):
     """The schedule restated with eager PyTorch on the host cores (the CPU oracle), on a bounded sample.  This leg is
     the only place where the bench touches the oracle: it times it and, with ``sampled = (x rows, W_gate, W_up,
-    W_down, {name: the GPU result's same rows})``, checks the timed GPU results against its fp32 evaluation."""
+    W_down, {name: the GPU result's same rows})``, checks the timed GPU results against its fp32 evaluation;
+    ``other_checks``: {configuration: callable(oracle modules) -> error figures} for the other configurations'
+    sampled rows.  ``time_it`` False: only those checks (returned as they are)."""
+    from oracle import decode as oracle_decode
+    from oracle import decoder as oracle_decoder
     from oracle import mlp as oracle_mlp
 
+    modules = {"mlp": oracle_mlp, "decoder": oracle_decoder, "decode": oracle_decode}
+    others = {name: check(modules) for name, check in (other_checks or {}).items() if check is not None}
+    if not time_it:
+        return others
     checks = {}
     if sampled is not None:
         x_rows, wg_s, wu_s, wd_s, got = sampled
@@ -735,6 +909,7 @@ def cpu_baseline(torch, sampled=None):
     c1_median = c1_times[len(c1_times) // 2]
     return {
         "gpu_results_rel_err_vs_fp32_oracle_sampled_rows": checks,
+        "other_configs_rel_err_vs_oracle_sampled_rows": others,
         "value": sample_tokens / median,
         "unit": "tokens/s",
         "cores": torch.get_num_threads(),
@@ -753,6 +928,42 @@ def cpu_baseline(torch, sampled=None):
     }
 
 
+#: the issue mode that `value` is measured in (fixed, not the best of several): one stream per nano-batch, the
+#: gate/up GEMM with the SiLU*mul as its epilogue, kernels planned for the two launches of a kind that run side by
+#: side (the manager derives that from the stream policy), the whole two-stream schedule as one hipGraph
+HEADLINE_KNOBS = {"whole_graph": True, "fuse_silu_epilogue": True, "streams": "by_nano_batch"}
+HEADLINE_MODE = "overlapped_hipgraph+silu_mul_epilogue+staggered+stream_per_nano_batch+kernels_planned_for_the_pair"
+
+
+def headline_workload(mb):
+    return (f"Llama-3-8B-shaped SwiGLU MLP layer, x[{TOKENS},{HIDDEN}] bf16 pre-normed, I={INTER}, {SPLITS} "
+            f"nano-batches of {mb} tokens, each on a HIP stream of its own: per nano-batch ONE launch for the gate "
+            "and up projections with the SiLU*mul as its epilogue, then the down projection; the two nano-batches' "
+            "launches of the same kind run side by side (the gate/up/SiLU launch of nano-batch 1 beside that of "
+            "nano-batch 0, then the two down projections) with kernels planned for the pair; the whole two-stream "
+            "schedule replayed as one hipGraph")
+
+
+def other_configs(torch, args):
+    """The other three GPU configurations with few steps each, for the one default line: (name, figures, check)
+    with ``check(oracle modules) -> error of sampled rows`` run later by the CPU leg."""
+    out, checks = {}, {}
+    steps, warmup = max(5, args.steps // 4), max(3, args.warmup // 2)
+    for name, fn in (("decoder_layer_prefill_8x2048", decoder_config), ("fp8_mlp_70b_shape", fp8_config),
+                     ("decode_step_32_layers", decode_config)):
+        print(f"bench.py: other configuration {name}", file=sys.stderr, flush=True)
+        line = fn(torch, steps, warmup, brief=True)
+        checks[name] = line.pop("oracle_check", None)
+        out[name] = {k: line[k] for k in ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "dtype", "config",
+                                          "roofline", "timings") if k in line}
+        for extra in ("layer", "overlap_speedup"):
+            if extra in line:
+                out[name][extra] = line[extra]
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+    return out, checks
+
+
 def main() -> int:
     args = parse_args()
     read_knobs(args.knob)
@@ -769,12 +980,15 @@ def main() -> int:
 
     _cabi.load()
     info = _cabi.device_info(0)
-    if args.decoder:
-        print(json.dumps(decoder_config(torch, max(5, args.steps // 5), max(3, args.warmup // 5))))
-        return 0
-    if args.decode:
-        print(json.dumps(decode_config(torch, max(5, args.steps // 5), max(3, args.warmup // 5))))
-        return 0
+    single = [(args.decoder, decoder_config), (args.decode, decode_config), (args.fp8, fp8_config)]
+    for wanted, fn in single:
+        if wanted:
+            line = fn(torch, max(5, args.steps // 5), max(3, args.warmup // 5))
+            check = line.pop("oracle_check", None)
+            if check is not None and not args.skip_cpu:
+                line["rel_err_vs_oracle_sampled_rows"] = cpu_baseline(torch, None, {"this": check}, time_it=False)["this"]
+            print(json.dumps(line))
+            return 0
     if args.decode_kernels:
         line = decode_kernels(torch, ops, max(20, args.steps))
         line["projections"] = decode_projections(torch, ops, max(20, args.steps))
@@ -782,9 +996,6 @@ def main() -> int:
         return 0
     if args.prefill_attention_kernels:
         print(json.dumps(prefill_attention_kernels(torch, ops, max(20, args.steps))))
-        return 0
-    if args.fp8:
-        print(json.dumps(fp8_config(torch, max(5, args.steps // 5), max(3, args.warmup // 5))))
         return 0
     x_cpu, wg, wu, wd = synthetic_inputs(torch, TOKENS, HIDDEN, INTER, torch.bfloat16)
     x = x_cpu.cuda()
@@ -794,118 +1005,158 @@ def main() -> int:
         print(json.dumps(single_kernels(torch, ops, x, weights, max(20, args.steps), calibration_copy=True)))
         return 0
 
+    settle = args.settle_seconds
     if args.headline_only:
-        m_h, c_h = build_path(torch, x, weights, whole_graph=True, fuse_silu_epilogue=True)
-        ms_h, _ = time_steps(torch, m_h, c_h, x, args.steps, args.warmup, use_graph=True)
-        print(json.dumps({"mode": "overlapped_hipgraph+silu_mul_epilogue", "ms_per_step": ms_h, "steps": args.steps}))
+        m_h, c_h = build_path(torch, x, weights, **HEADLINE_KNOBS)
+        ms_h, _ = time_steps(torch, m_h, c_h, x, args.steps, args.warmup, use_graph=True, settle_s=settle)
+        print(json.dumps({"mode": HEADLINE_MODE, "ms_per_step": ms_h, "steps": args.steps}))
         return 0
 
-    # ---- the ways of issuing the schedule (serialized: every launch on one stream, eagerly and as one graph)
+    mb = TOKENS // SPLITS
+    # ---- the headline mode first: straight after its set-up (the GPU has idled through the trace), then with the
+    # package settled - every timed loop of this run is preceded by `settle` seconds of the same step, untimed, so
+    # that the modes are compared in one state of the clocks; W warm-up steps and exactly K timed steps follow
+    m_head, c_head = build_path(torch, x, weights, **HEADLINE_KNOBS)
+    assert m_head.launches_side_by_side(m_head.prepare(TOKENS, [TOKENS])) == SPLITS
+    ms_head_from_idle, _ = time_steps(torch, m_head, c_head, x, args.steps, args.warmup, use_graph=True)
+    ms_head, y_head = time_steps(torch, m_head, c_head, x, args.steps, args.warmup, use_graph=True, settle_s=settle)
+    y_head = y_head.clone()
+    load_s = args.sustain_seconds
+    ms_sustained = sustained_steps(torch, m_head, c_head, x, args.steps, load_s) if load_s > 0 else None
+    # the same kernels and the same split on ONE stream, as one graph: the baseline of `overlap_speedup`
+    m_h1, c_h1 = build_path(torch, x, weights, serialize=True, whole_graph=True, fuse_silu_epilogue=True,
+                            side_by_side=SPLITS)
+    ms_head_one_stream, y_head_one_stream = time_steps(torch, m_h1, c_h1, x, args.steps, args.warmup, use_graph=True,
+                                                       settle_s=settle)
+    head_identical = bool(torch.equal(y_head, y_head_one_stream))
+
+    # ---- separate kernels (gate GEMM, up GEMM, SiLU*mul, down GEMM): every launch on one stream, eagerly and as one
+    # graph; then the north star's own pattern - streams by sub-graph kind, staggered: the gate/up GEMMs of nano-batch
+    # 1 beside SiLU*mul + down projection of nano-batch 0
     m_ser, c_ser = build_path(torch, x, weights, serialize=True, whole_graph=True)
-    ms_serial, y_serial = time_steps(torch, m_ser, c_ser, x, args.steps, args.warmup, use_graph=False)
+    ms_serial, y_serial = time_steps(torch, m_ser, c_ser, x, args.steps, args.warmup, use_graph=False, settle_s=settle)
     y_serial = y_serial.clone()
     ms_serial_gpu = gpu_time_of_steps(torch, m_ser, c_ser, x, min(args.steps, 20))
-    ms_serial_graph, y_serial_graph = time_steps(torch, m_ser, c_ser, x, args.steps, args.warmup, use_graph=True)
+    ms_serial_graph, y_serial_graph = time_steps(torch, m_ser, c_ser, x, args.steps, args.warmup, use_graph=True,
+                                                 settle_s=settle)
     serial_graph_identical = bool(torch.equal(y_serial, y_serial_graph))
     m_ovl, c_ovl = build_path(torch, x, weights, whole_graph=True)
-    ms_eager, y_eager = time_steps(torch, m_ovl, c_ovl, x, args.steps, args.warmup, use_graph=False)
+    ms_eager, y_eager = time_steps(torch, m_ovl, c_ovl, x, args.steps, args.warmup, use_graph=False, settle_s=settle)
     y_eager = y_eager.clone()
-    ms_graph, y_graph = time_steps(torch, m_ovl, c_ovl, x, args.steps, args.warmup, use_graph=True)
+    ms_graph, y_graph = time_steps(torch, m_ovl, c_ovl, x, args.steps, args.warmup, use_graph=True, settle_s=settle)
     identical = bool(torch.equal(y_serial, y_eager) and torch.equal(y_eager, y_graph))
     y_graph = y_graph.clone()
-    # the same separate kernels with one stream per nano-batch and the kernels planned for the pair (see the fused
-    # modes below): the two nano-batches' launches of each kind run side by side
-    m_op, c_op = build_path(torch, x, weights, whole_graph=True, streams="by_nano_batch", side_by_side=2)
-    ms_graph_pair, y_graph_pair = time_steps(torch, m_op, c_op, x, args.steps, args.warmup, use_graph=True)
+    # the same separate kernels with one stream per nano-batch, planned for the pair
+    m_op, c_op = build_path(torch, x, weights, whole_graph=True, streams="by_nano_batch")
+    ms_graph_pair, y_graph_pair = time_steps(torch, m_op, c_op, x, args.steps, args.warmup, use_graph=True,
+                                             settle_s=settle)
     y_graph_pair = y_graph_pair.clone()
-    m_ops, c_ops = build_path(torch, x, weights, serialize=True, side_by_side=2)
+    m_ops, c_ops = build_path(torch, x, weights, serialize=True, side_by_side=SPLITS)
     _, y_serial_pair = time_steps(torch, m_ops, c_ops, x, 2, 1, use_graph=False)
     pair_identical = bool(torch.equal(y_serial_pair, y_graph_pair))
 
-    # ---- the same layer with the SiLU*mul as the epilogue of one gate/up GEMM
+    # ---- the SiLU*mul as the epilogue of one gate/up GEMM, in the other issue modes
     m_fs, c_fs = build_path(torch, x, weights, serialize=True, whole_graph=True, fuse_silu_epilogue=True)
-    ms_fused_serial, yf_serial = time_steps(torch, m_fs, c_fs, x, args.steps, args.warmup, use_graph=False)
+    ms_fused_serial, yf_serial = time_steps(torch, m_fs, c_fs, x, args.steps, args.warmup, use_graph=False,
+                                            settle_s=settle)
     yf_serial = yf_serial.clone()
     ms_fused_serial_gpu = gpu_time_of_steps(torch, m_fs, c_fs, x, min(args.steps, 20))
-    ms_fused_serial_graph, _ = time_steps(torch, m_fs, c_fs, x, args.steps, args.warmup, use_graph=True)
+    ms_fused_serial_graph, _ = time_steps(torch, m_fs, c_fs, x, args.steps, args.warmup, use_graph=True,
+                                          settle_s=settle)
+    # the north star's pattern again (streams by kind, staggered): the fused GEMM of nano-batch 1 beside the down
+    # projection of nano-batch 0
     m_fo, c_fo = build_path(torch, x, weights, whole_graph=True, fuse_silu_epilogue=True)
-    ms_fused_graph, yf_graph = time_steps(torch, m_fo, c_fo, x, args.steps, args.warmup, use_graph=True)
-    fused_identical = bool(torch.equal(yf_serial, yf_graph))
+    ms_fused_graph, yf_graph = time_steps(torch, m_fo, c_fo, x, args.steps, args.warmup, use_graph=True,
+                                          settle_s=settle)
     yf_graph = yf_graph.clone()
-    # the same kernels in the order that issues both nano-batches' launches against the same weights back to back
-    # (gate/up/SiLU of nano-batch 0 and 1, then the two down projections): the second launch of a pair finds most of
-    # the weights in the memory-side cache.  Two ways to get that order: the round-robin schedule (the NanoFlow
-    # order of the reference), or one stream per nano-batch (the second gate/up/SiLU launch is queued while the first
-    # holds the compute units)
-    m_fn, c_fn = build_path(torch, x, weights, whole_graph=True, fuse_silu_epilogue=True, streams="by_nano_batch")
-    ms_fused_graph_nb, yf_graph_nb = time_steps(torch, m_fn, c_fn, x, args.steps, args.warmup, use_graph=True)
+    # weights-major orders (both nano-batches' launches against the same weights back to back; the second finds most
+    # of them in the memory-side cache), kernels planned as lone launches: one stream per nano-batch, or the
+    # round-robin schedule (the NanoFlow order of the reference)
+    m_fn, c_fn = build_path(torch, x, weights, whole_graph=True, fuse_silu_epilogue=True, streams="by_nano_batch",
+                            side_by_side=1)
+    ms_fused_graph_nb, yf_graph_nb = time_steps(torch, m_fn, c_fn, x, args.steps, args.warmup, use_graph=True,
+                                                settle_s=settle)
+    yf_graph_nb = yf_graph_nb.clone()
     m_fr, c_fr = build_path(torch, x, weights, whole_graph=True, fuse_silu_epilogue=True, schedule="round_robin")
-    ms_fused_graph_rr, yf_graph_rr = time_steps(torch, m_fr, c_fr, x, args.steps, args.warmup, use_graph=True)
-    fused_identical = (fused_identical and bool(torch.equal(yf_serial, yf_graph_nb))
-                       and bool(torch.equal(yf_serial, yf_graph_rr)))
-    # one stream per nano-batch, and the kernels planned for two launches side by side: the down projections (128
-    # tiles of 256 x 256 each) with one workgroup per tile instead of K split over two - together they fill the 256
-    # compute units and need no fp32 hand-over - and the gate/up/SiLU launches with the 256 x (128 + 128) tile
-    # (2 x 896 tiles are exactly 7 rounds).  Other additions than with K split: not the same bits, checked
-    # against the oracle like the others
-    m_fu, c_fu = build_path(torch, x, weights, whole_graph=True, fuse_silu_epilogue=True, streams="by_nano_batch",
-                            side_by_side=2)
-    ms_fused_graph_nb_unsplit, yf_graph_nbu = time_steps(torch, m_fu, c_fu, x, args.steps, args.warmup, use_graph=True)
-    yf_graph_nbu = yf_graph_nbu.clone()
-    m_fus, c_fus = build_path(torch, x, weights, serialize=True, fuse_silu_epilogue=True, side_by_side=2)
-    _, yf_serial_unsplit = time_steps(torch, m_fus, c_fus, x, 2, 1, use_graph=False)
-    unsplit_identical = bool(torch.equal(yf_serial_unsplit, yf_graph_nbu))
-    fused_modes = {"+staggered+streams_by_sub_graph_kind": (ms_fused_graph, m_fo, c_fo, yf_graph),
-                   "+staggered+stream_per_nano_batch": (ms_fused_graph_nb, m_fn, c_fn, yf_graph),
-                   "+round_robin+streams_by_sub_graph_kind": (ms_fused_graph_rr, m_fr, c_fr, yf_graph),
-                   "+staggered+stream_per_nano_batch+kernels_planned_for_the_pair": (ms_fused_graph_nb_unsplit, m_fu, c_fu,
-                                                                          yf_graph_nbu)}
-    best_fused_mode = min(fused_modes, key=lambda m: fused_modes[m][0])
-    ms_fused_best = fused_modes[best_fused_mode][0]
+    ms_fused_graph_rr, yf_graph_rr = time_steps(torch, m_fr, c_fr, x, args.steps, args.warmup, use_graph=True,
+                                                settle_s=settle)
+    yf_graph_rr = yf_graph_rr.clone()
+    fused_identical = all(bool(torch.equal(yf_serial, other)) for other in (yf_graph, yf_graph_nb, yf_graph_rr))
+    fused_modes = {"+staggered+streams_by_sub_graph_kind": (ms_fused_graph, yf_graph),
+                   "+staggered+stream_per_nano_batch": (ms_fused_graph_nb, yf_graph_nb),
+                   "+round_robin+streams_by_sub_graph_kind": (ms_fused_graph_rr, yf_graph_rr),
+                   "+staggered+stream_per_nano_batch+kernels_planned_for_the_pair": (ms_head, y_head)}
+    fastest_fused_mode = min(fused_modes, key=lambda m: fused_modes[m][0])
 
     # ---- for comparison only: the 4096 tokens as ONE batch (no nano-batches, one stream, two launches)
     m_un, c_un = build_path(torch, x, weights, min_nano_split_tokens=1 << 30, fuse_silu_epilogue=True)
     ms_unsplit_gpu = gpu_time_of_steps(torch, m_un, c_un, x, min(args.steps, 20))
 
+    if not (head_identical and fused_identical and identical and serial_graph_identical and pair_identical):
+        print("bench.py: issue modes that run the same kernels disagree bit for bit: "
+              f"headline vs its one-stream issue {head_identical}, fused modes {fused_identical}, separate kernels "
+              f"{identical and serial_graph_identical}, pair plan {pair_identical}", file=sys.stderr)
+        return 1
+
     # ---- sampled rows of the timed results, checked against the fp32 oracle (same bf16 operands) in the CPU leg
     rows = torch.tensor([0, 2047, 2048, 4095])
-    y_best_fused = fused_modes[best_fused_mode][3]
     sampled = (x_cpu[rows], wg, wu, wd, {"separate_kernels_graph": y_graph[rows].float().cpu(),
-                                         "best_fused_mode": y_best_fused[rows].float().cpu()})
+                                         "headline_mode": y_head[rows].float().cpu(),
+                                         "fused_lone_plans": yf_graph[rows].float().cpu()})
 
     # ---- single kernels, HIP events on the launching stream
     k = single_kernels(torch, ops, x, weights, max(20, args.steps))
     ms_gate, ms_down, ms_silu, ms_blas = k["gate_ms"], k["down_ms"], k["silu_ms"], k["blas_ms"]
     ms_gus = k["gate_up_silu_ms"]
     ms_gus_pair, ms_down_pair = k["gate_up_silu_pair_ms"], k["down_pair_ms"]
-    mb = TOKENS // SPLITS
     gemm_flops = 2.0 * mb * HIDDEN * INTER          # one projection of one nano-batch
     silu_bytes = 3.0 * mb * INTER * 2               # read gate + up, write out
     layer_flops = 6.0 * TOKENS * HIDDEN * INTER
 
-    fused_wins = ms_fused_best < ms_graph
-    best_ms = ms_fused_best if fused_wins else ms_graph
     result = {
         "metric": METRIC,
-        "value": TOKENS / (best_ms * 1e-3),
+        "value": TOKENS / (ms_head * 1e-3),
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": best_ms,
+        "ms_per_step": ms_head,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": f"Llama-3-8B-shaped SwiGLU MLP layer, x[{TOKENS},{HIDDEN}] bf16 pre-normed, I={INTER}, "
-                        f"{SPLITS} nano-batches of {mb}, gate/up GEMM of nano-batch 1 beside SiLU*mul+down of "
-                        "nano-batch 0 on two HIP streams, whole schedule replayed as one hipGraph",
-            "issue_mode": "overlapped_hipgraph" + ("+silu_mul_epilogue" + best_fused_mode if fused_wins
-                                                   else "+silu_mul_kernel+staggered+streams_by_sub_graph_kind"),
+            "workload": headline_workload(mb),
+            "issue_mode": HEADLINE_MODE,
             "device": info["arch_name"],
             "compute_units": info["compute_units"],
+            # every timed loop: `settle` seconds of the same step untimed (clocks of the package in their loaded
+            # state), then W warm-up steps, then exactly K timed steps between two device synchronisations
+            "settle_seconds_before_each_timed_loop": settle,
+            "ms_per_step_straight_after_set_up": ms_head_from_idle,
+        },
+        # the overlap figure of the measurement plan: the same kernels and the same split issued on one stream against
+        # the two-stream schedule, both replayed as one hipGraph
+        "overlap_speedup": ms_head_one_stream / ms_head,
+        "overlap_speedup_parts": {
+            "one_stream_same_kernels_graph_ms": ms_head_one_stream,
+            "two_streams_graph_ms": ms_head,
+            "what_runs_side_by_side": "launches of the same kind: gate/up/SiLU of both nano-batches, then both down "
+                                      "projections (a lone launch of these plans fills half the compute units)",
+            # the one-stream schedule in ITS best form (kernels planned as lone launches)
+            "one_stream_lone_plans_graph_ms": ms_fused_serial_graph,
+            "speedup_vs_one_stream_lone_plans_graph": ms_fused_serial_graph / ms_head,
+            "outputs_bit_identical_to_the_one_stream_issue": head_identical,
+        },
+        # the pattern the north star names - streams by sub-graph kind, staggered: the GEMM sub-graph of nano-batch 1
+        # beside SiLU*mul + down projection of nano-batch 0 - against the same kernels on one stream, graph vs graph
+        "north_star_pattern_gemm_beside_tail_of_previous_nano_batch": {
+            "separate_silu_mul_kernel": {"one_stream_graph_ms": ms_serial_graph, "two_streams_graph_ms": ms_graph,
+                                         "speedup": ms_serial_graph / ms_graph},
+            "silu_mul_as_gemm_epilogue": {"one_stream_graph_ms": ms_fused_serial_graph,
+                                          "two_streams_graph_ms": ms_fused_graph,
+                                          "speedup": ms_fused_serial_graph / ms_fused_graph},
         },
         # reported beside the nano-batch schedule, never as `value`: every operator of this layer is MFMA-bound, so
         # on one GPU two nano-batches have nothing of a different kind to hide behind each other
@@ -932,21 +1183,20 @@ def main() -> int:
             "overlapped_graph_ms": ms_fused_graph,
             "overlapped_graph_stream_per_nano_batch_ms": ms_fused_graph_nb,
             "overlapped_graph_round_robin_ms": ms_fused_graph_rr,
-            "overlapped_graph_stream_per_nano_batch_planned_for_the_pair_ms": ms_fused_graph_nb_unsplit,
+            "overlapped_graph_stream_per_nano_batch_planned_for_the_pair_ms": ms_head,
             "speedup_graph_vs_serialized": ms_fused_serial / ms_fused_graph,
             "speedup_graph_vs_serialized_gpu_side": ms_fused_serial_gpu / ms_fused_graph,
             "speedup_graph_vs_serialized_graph": ms_fused_serial_graph / ms_fused_graph,
-            "best_mode": best_fused_mode[1:],
-            "best_graph_ms": ms_fused_best,
-            # against the one-stream issue in its own best form (kernels planned for lone launches)
-            "speedup_best_vs_serialized": ms_fused_serial / ms_fused_best,
-            "speedup_best_vs_serialized_graph": ms_fused_serial_graph / ms_fused_best,
+            "fastest_mode_of_this_run": fastest_fused_mode[1:],
+            "headline_mode_ms": ms_head,
+            "speedup_headline_vs_serialized": ms_fused_serial / ms_head,
+            "speedup_headline_vs_serialized_graph": ms_fused_serial_graph / ms_head,
             "outputs_bit_identical": fused_identical,
-            "planned_for_the_pair_bit_identical_to_its_serialized_issue": unsplit_identical,
+            "planned_for_the_pair_bit_identical_to_its_serialized_issue": head_identical,
         },
         "layer": {
-            "tflops": layer_flops / (best_ms * 1e-3) / 1e12,
-            "frac_of_bf16_mfma_peak": layer_flops / (best_ms * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
+            "tflops": layer_flops / (ms_head * 1e-3) / 1e12,
+            "frac_of_bf16_mfma_peak": layer_flops / (ms_head * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
         },
         "kernels": {
             "gate_or_up_gemm": {"ms": ms_gate, "tflops": gemm_flops / (ms_gate * 1e-3) / 1e12},
@@ -974,85 +1224,69 @@ def main() -> int:
         },
         # the layer the same way: separate GEMM and SiLU*mul launches of both nano-batches one after the other on
         # one stream (the reference's serial baseline) against the issue mode that `value` comes from
-        "speedup_best_vs_serialized_separate_kernels": ms_serial / best_ms,
-        "speedup_best_vs_serialized_separate_kernels_graph": ms_serial_graph / best_ms,
+        "speedup_best_vs_serialized_separate_kernels": ms_serial / ms_head,
+        "speedup_best_vs_serialized_separate_kernels_graph": ms_serial_graph / ms_head,
     }
     # the dominant kernel of the issue mode that `value` comes from
-    if fused_wins and best_fused_mode.endswith("kernels_planned_for_the_pair"):
-        result["roofline"] = {
-            "kernel": "gemm_bf16_ring_kernel<true> (gate and up projection of one nano-batch with the SiLU*mul epilogue, "
-                      "256 x (128 + 128) tile: [2048,4096] x 2 x [14336,4096]^T -> act[2048,14336]); the two "
-                      "nano-batches' launches run side by side on two streams and are timed as pairs (two loops of "
-                      "launches, one per stream)",
-            "bound": "mfma",
-            "achieved": 4 * gemm_flops / (ms_gus_pair * 1e-3) / 1e12,
-            "peak": BF16_MFMA_PEAK_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": 4 * gemm_flops / (ms_gus_pair * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
-            "launches_timed_together": 2,
-            # per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy of known size; algorithmic:
-            # 16.8 + 2 x 117.4 MB read, 58.7 MB written
-            "traffic": GATE_UP_SILU_SQUARE_TRAFFIC_BYTES,
-            "traffic_unit": "bytes per launch",
-        }
-    elif fused_wins:
-        result["roofline"] = {
-            "kernel": "gemm_bf16_gate_up_silu_walk_kernel (gate and up projection of one nano-batch with the SiLU*mul "
-                      "epilogue: [2048,4096] x 2 x [14336,4096]^T -> act[2048,14336])",
-            "bound": "mfma",
-            "achieved": 2 * gemm_flops / (ms_gus * 1e-3) / 1e12,
-            "peak": BF16_MFMA_PEAK_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": 2 * gemm_flops / (ms_gus * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
-            # HBM-side bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy of
-            # known size; algorithmic: 16.8 + 2 x 117.4 MB read, 58.7 MB written
-            "traffic": GATE_UP_SILU_TRAFFIC_BYTES,
-            "traffic_unit": "bytes per launch",
-        }
-    else:
-        result["roofline"] = {
-            "kernel": "gemm_bf16_ring224_kernel<false> (gate or up projection of one nano-batch: "
-                      "[2048,4096] x [14336,4096]^T)",
-            "bound": "mfma",
-            "achieved": gemm_flops / (ms_gate * 1e-3) / 1e12,
-            "peak": BF16_MFMA_PEAK_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": gemm_flops / (ms_gate * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
-            # algorithmic: 134.2 MB read + 58.7 MB written
-            "traffic": GATE_GEMM_TRAFFIC_BYTES,
-            "traffic_unit": "bytes per launch",
-        }
-    # ---- the same figures under sustained load (`value` stays the short-loop figure defined above)
-    load_s = args.sustain_seconds
+    result["roofline"] = {
+        "kernel": GATE_UP_SILU_PAIR_KERNEL + " (gate and up projection of one nano-batch with the SiLU*mul epilogue: "
+                  "[2048,4096] x 2 x [14336,4096]^T -> act[2048,14336]); the two nano-batches' launches run side by "
+                  "side on two streams and are timed as pairs (two loops of launches, one per stream)",
+        "bound": "mfma",
+        "achieved": 4 * gemm_flops / (ms_gus_pair * 1e-3) / 1e12,
+        "peak": BF16_MFMA_PEAK_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": 4 * gemm_flops / (ms_gus_pair * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
+        "launches_timed_together": 2,
+        # per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy of known size; algorithmic:
+        # 16.8 + 2 x 117.4 MB read, 58.7 MB written
+        "traffic": GATE_UP_SILU_SQUARE_TRAFFIC_BYTES,
+        "traffic_unit": "bytes per launch",
+    }
+    # ---- the same figures under sustained load
     if load_s > 0:
-        m_best, c_best = fused_modes[best_fused_mode][1:3] if fused_wins else (m_ovl, c_ovl)
-        ms_sustained = sustained_steps(torch, m_best, c_best, x, args.steps, load_s)
         mb_x = x[:mb]
+        halves = (x[:mb], x[mb:2 * mb])
         with torch.no_grad():
-            if fused_wins:
-                # (the lone-launch form of the gate/up/SiLU kernel, whichever form the best mode uses)
-                ms_k = sustained_kernel(torch, lambda: ops.gate_up_silu(mb_x, weights[0], weights[1]),
-                                        max(20, args.steps), load_s)
-                k_flops = 2 * gemm_flops
-            else:
-                ms_k = sustained_kernel(torch, lambda: ops.linear(mb_x, weights[0]), max(20, args.steps), load_s)
-                k_flops = gemm_flops
+            def pair_of(i):
+                with ops.launch_options(side_by_side=SPLITS):
+                    return ops.gate_up_silu(halves[i], weights[0], weights[1])
+
+            until = time.perf_counter() + load_s
+            while time.perf_counter() < until:
+                for _ in range(50):
+                    ops.gate_up_silu(mb_x, weights[0], weights[1])
+                torch.cuda.synchronize()
+            ms_k_pair = time_pair(torch, pair_of, max(20, args.steps), warmup=5)
         result["sustained"] = {
-            "method": f"the same graph replay / the same kernel launch timed right after {load_s:g} s of running "
-                      "it back to back (package at its power limit, clocks settled)",
+            "method": f"the same graph replay / the same pair of launches timed right after {load_s:g} s of running "
+                      "the step / the kernel back to back (package at its power limit, clocks settled)",
             "load_seconds": load_s,
             "ms_per_step": ms_sustained,
             "value": TOKENS / (ms_sustained * 1e-3),
             "layer_frac_of_bf16_mfma_peak": layer_flops / (ms_sustained * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
-            "dominant_kernel_ms": ms_k,
-            "dominant_kernel_frac": k_flops / (ms_k * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
+            "dominant_kernel_pair_ms": ms_k_pair,
+            "dominant_kernel_frac": 4 * gemm_flops / (ms_k_pair * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
         }
+    checks = {}
+    if not args.headline_config_only:
+        del m_head, c_head, m_h1, c_h1, m_ser, c_ser, m_ovl, c_ovl, m_op, c_op, m_ops, c_ops, m_fs, c_fs, m_fo, c_fo
+        del m_fn, c_fn, m_fr, c_fr, m_un, c_un, weights, x
+        torch.cuda.empty_cache()
+        result["other_configs"], checks = other_configs(torch, args)
     if not args.skip_cpu:
-        result["cpu_baseline"] = cpu_baseline(torch, sampled)
+        result["cpu_baseline"] = cpu_baseline(torch, sampled, checks)
         worst = max(result["cpu_baseline"]["gpu_results_rel_err_vs_fp32_oracle_sampled_rows"].values())
         if not worst < 2e-2:
             print(f"bench.py: the timed result is off the fp32 oracle by {worst:.3g} (bf16 bound 2e-2)", file=sys.stderr)
             return 1
+        for name, err in result["cpu_baseline"].pop("other_configs_rel_err_vs_oracle_sampled_rows", {}).items():
+            result["other_configs"][name]["rel_err_vs_oracle_sampled_rows"] = err
+            bound = 5e-2 if "fp8" in name else 0.1 if "decode_step" in name else 2e-2
+            if not err["worst"] < bound:
+                print(f"bench.py: {name}: sampled rows are off the oracle by {err['worst']:.3g} (bound {bound})",
+                      file=sys.stderr)
+                return 1
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))

@@ -238,7 +238,7 @@ class DynaFlowManager:
 
         from dynaflow_amd import ops
 
-        with ops.launch_options(side_by_side=int(self.config.knob("side_by_side", 1))):
+        with ops.launch_options(side_by_side=self.launches_side_by_side(split)):
             if split.is_dryrun:
                 results, events = self.engine.dryrun(args, kwargs, split)
             else:
@@ -250,6 +250,40 @@ class DynaFlowManager:
         for event in events:
             event.wait()
         return join_results(results, len(results), getattr(self.engine, "shared_output_buffer", None))
+
+    def launches_side_by_side(self, split: SplitConfig) -> int:
+        """How many nano-batches run the SAME sub-graph at the same time in a forward with this split - what the
+        kernel plans are made for (``ops.launch_options``).  It follows from the schedule, not from a promise of
+        the user: the shipped schedulers pick a launch's stream from the sub-graph's tag (``streams="by_kind"``,
+        the reference's policies, examples/ae/scheduler/hf/nanoflow.py:122-146: launches of one kind queue on one
+        stream, so a launch of a kind runs alone) or from the nano-batch (``"by_nano_batch"``: two streams that the
+        nano-batches take in turn, so two nano-batches run the same sub-graph side by side); one stream
+        (``serialize``), one nano-batch, or a scheduler that does not say how it assigns streams give 1.
+
+        ``additional_config["side_by_side"]`` overrides the derived figure downwards (kernels planned as for
+        fewer co-runners, for comparisons); a figure above it contradicts the schedule - launches planned for
+        partners that never run - and is refused, except on the one-stream schedule, which is the baseline of
+        whichever plan it is given (same kernels, nothing overlapped)."""
+        assert self.config is not None and self.scheduler is not None
+        lanes = split.num_nano_batches
+        if split.is_dryrun:      # a dry-run captures what the scheduled forwards replay: plan as for those
+            lanes = int(getattr(self.scheduler, "num_nano_batches", self.config.max_num_splits))
+        policy = getattr(self.scheduler, "stream_policy", None)
+        main, side = getattr(self.scheduler, "comp_stream", None), getattr(self.scheduler, "comm_stream", None)
+        one_stream = main is None or main is side
+        derived = min(lanes, 2) if (policy == "by_nano_batch" and not one_stream) else 1
+        asked = self.config.knob("side_by_side", None)
+        if asked is None or asked == "auto":
+            return derived
+        asked = int(asked)
+        if asked < 1:
+            raise ValueError(f"side_by_side={asked}: at least one launch runs")
+        if asked > derived and not one_stream:
+            raise ValueError(
+                f"side_by_side={asked} contradicts the schedule: with streams={policy!r} and {lanes} nano-batch(es) "
+                f"{derived} launch(es) of a sub-graph run at the same time; leave the knob out (it is derived) or "
+                'use streams="by_nano_batch"')
+        return asked
 
     # ------------------------------------------------- whole-schedule graphs
     def _wants_whole_graph(self, split: SplitConfig) -> bool:

@@ -40,30 +40,37 @@ def attend(q: torch.Tensor, keys: torch.Tensor, values: torch.Tensor) -> torch.T
     return out
 
 
+def decode_layer(x, slots, lengths, params, i, k_cache, v_cache, heads, kv_heads, theta=500000.0, eps=1e-5):
+    """Layer ``i`` of the step on hidden states ``x [T, hidden]`` (float64): attention block, then MLP block.
+    ``k_cache`` / ``v_cache``: that layer's caches, float64 ``[slots, capacity, kv_heads, d]``, updated in place
+    (token t's key and value go to position ``lengths[t] - 1`` of slot ``slots[t]``).  Returns ``[T, hidden]``."""
+    d = k_cache.shape[-1]
+    T = x.shape[0]
+    pos = lengths.long() - 1
+    h = rms_norm(x, params[f"attn_norm.{i}"], eps)
+    qkv = h @ params[f"wqkv.{i}"].t()
+    q = rope_at(qkv[:, : heads * d].reshape(T, heads, d), pos, theta)
+    k = rope_at(qkv[:, heads * d: (heads + kv_heads) * d].reshape(T, kv_heads, d), pos, theta)
+    v = qkv[:, (heads + kv_heads) * d:].reshape(T, kv_heads, d)
+    attn = torch.empty(T, heads * d, dtype=torch.float64)
+    for t in range(T):
+        s, L = int(slots[t]), int(lengths[t])
+        k_cache[s, L - 1] = k[t]
+        v_cache[s, L - 1] = v[t]
+        attn[t] = attend(q[t], k_cache[s, :L], v_cache[s, :L]).reshape(-1)
+    x = x + attn @ params[f"wo.{i}"].t()
+    h = rms_norm(x, params[f"mlp_norm.{i}"], eps)
+    g = h @ params[f"w_gate.{i}"].t()
+    return x + ((g / (1 + torch.exp(-g))) * (h @ params[f"w_up.{i}"].t())) @ params[f"w_down.{i}"].t()
+
+
 def decode_step(token_ids, slots, lengths, params, k_caches, v_caches, heads, kv_heads, theta=500000.0, eps=1e-5):
     """One new token per sequence.  ``params``: dict with ``embed`` and per layer i ``attn_norm.i``, ``wqkv.i``,
     ``wo.i``, ``mlp_norm.i``, ``w_gate.i``, ``w_up.i``, ``w_down.i`` (float64).  ``k_caches[i]`` /
     ``v_caches[i]``: float64 ``[slots, capacity, kv_heads, d]``, updated in place.  Returns ``[T, hidden]``."""
-    d = k_caches[0].shape[-1]
     x = params["embed"][token_ids.long()]
-    T = x.shape[0]
-    pos = lengths.long() - 1
     for i in range(len(k_caches)):
-        h = rms_norm(x, params[f"attn_norm.{i}"], eps)
-        qkv = h @ params[f"wqkv.{i}"].t()
-        q = rope_at(qkv[:, : heads * d].reshape(T, heads, d), pos, theta)
-        k = rope_at(qkv[:, heads * d: (heads + kv_heads) * d].reshape(T, kv_heads, d), pos, theta)
-        v = qkv[:, (heads + kv_heads) * d:].reshape(T, kv_heads, d)
-        attn = torch.empty(T, heads * d, dtype=torch.float64)
-        for t in range(T):
-            s, L = int(slots[t]), int(lengths[t])
-            k_caches[i][s, L - 1] = k[t]
-            v_caches[i][s, L - 1] = v[t]
-            attn[t] = attend(q[t], k_caches[i][s, :L], v_caches[i][s, :L]).reshape(-1)
-        x = x + attn @ params[f"wo.{i}"].t()
-        h = rms_norm(x, params[f"mlp_norm.{i}"], eps)
-        g = h @ params[f"w_gate.{i}"].t()
-        x = x + ((g / (1 + torch.exp(-g))) * (h @ params[f"w_up.{i}"].t())) @ params[f"w_down.{i}"].t()
+        x = decode_layer(x, slots, lengths, params, i, k_caches[i], v_caches[i], heads, kv_heads, theta, eps)
     return x
 
 

@@ -415,3 +415,58 @@ def test_listed_sizes_get_their_own_callable_in_a_dry_run(host_device):
         y = compiled(x)
     torch.testing.assert_close(y, model(x), rtol=0, atol=0)
     assert calls == {"sized": 0, "dynamic": 2 * len(backends)}
+
+
+@pytest.mark.parametrize("knobs,splits,want", [
+    ({"streams": "by_nano_batch"}, 2, 2),                        # the same sub-graph of both nano-batches at once
+    ({"streams": "by_nano_batch"}, 4, 2),                        # four nano-batches take the two streams in turn
+    ({"streams": "by_kind"}, 2, 1),                              # launches of one kind queue on one stream
+    ({"streams": "by_nano_batch", "serialize": True}, 2, 1),     # one stream
+    ({"streams": "by_nano_batch", "side_by_side": 1}, 2, 1),     # override downwards: planned as lone launches
+    ({"streams": "by_kind", "serialize": True, "side_by_side": 2}, 2, 2),   # the one-stream baseline of a pair plan
+])
+def test_kernel_plans_follow_the_schedule_not_a_promise(host_device, monkeypatch, knobs, splits, want):
+    """``side_by_side`` - how many launches of one sub-graph share the GPU, what the GEMM plans are made for - is
+    derived from the stream policy and the split of each forward; the knob only overrides it downwards."""
+    import contextlib
+
+    from dynaflow_amd import ops
+
+    seen = []
+    real = ops.launch_options
+
+    @contextlib.contextmanager
+    def recording(side_by_side=1):
+        seen.append(side_by_side)
+        with real(side_by_side=side_by_side):
+            yield
+
+    monkeypatch.setattr(ops, "launch_options", recording)
+    cfg = make_config(splits, num_nano_batches=splits, **knobs)
+    model, manager, compiled, x = compile_mlp(cfg, tokens=96)
+    split = manager.prepare(96, [96])
+    assert split.num_nano_batches == splits
+    assert manager.launches_side_by_side(split) == want
+    seen.clear()
+    with torch.no_grad():
+        y = compiled(x)
+    assert seen == [want]
+    torch.testing.assert_close(y, model(x), rtol=0, atol=0)
+    # a forward that is not split has nothing beside it, whatever the stream policy
+    single = manager.prepare(4, [4])
+    assert single.num_nano_batches == 1
+    if "side_by_side" not in knobs:
+        assert manager.launches_side_by_side(single) == 1
+
+
+@pytest.mark.parametrize("knobs", [{"streams": "by_kind", "side_by_side": 2},
+                                   {"streams": "by_nano_batch", "side_by_side": 3},
+                                   {"streams": "by_nano_batch", "side_by_side": 0}])
+def test_a_side_by_side_override_that_contradicts_the_schedule_is_refused(host_device, knobs):
+    """Streams by sub-graph kind with kernels planned for a pair would queue two half-chip launches on one stream;
+    such a configuration raises instead of running slowly."""
+    cfg = make_config(2, num_nano_batches=2, **knobs)
+    model, manager, compiled, x = compile_mlp(cfg, tokens=96)
+    manager.prepare(96, [96])
+    with torch.no_grad(), pytest.raises(ValueError, match="side_by_side"):
+        compiled(x)

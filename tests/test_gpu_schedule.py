@@ -432,10 +432,15 @@ def test_listed_sizes_dispatch_to_their_own_lowered_callable():
 
 
 def test_fp8_config_full_size_properties():
-    """fp8 70B-shaped layer at full size (x[8192,8192], I=28672, 4 x 2048).  The CPU oracle cannot cover
-    this size in test time; the kernels are pinned on small shapes, here the schedule is: (1) the scheduled
-    two-stream run equals the nano-batches issued one after the other bit for bit, (2) two runs agree,
-    (3) sampled rows agree with an fp32 evaluation of the same quantised operands done with torch on the GPU."""
+    """fp8 70B-shaped layer at full size (x[8192,8192], I=28672, 4 x 2048), in both lowerings: separate gate / up /
+    SiLU*mul launches, and the mode the bench reports - gate, up, SiLU*mul and absmax as ONE launch
+    (``fuse_gate_up`` + knob ``fuse_silu_epilogue``).  (1) the scheduled two-stream run equals the nano-batches
+    issued one after the other bit for bit, (2) two runs agree, (3) the two lowerings agree bit for bit, (4) sampled
+    rows of two nano-batches agree with an evaluation that takes NOTHING from the kernels under test: activations
+    quantised with torch's own e4m3 conversion, gate and up of the WHOLE nano-batch as fp32 products of the
+    dequantised operands (torch on the GPU), rounded to bf16, the oracle's exact SiLU*mul, its absmax over the whole
+    nano-batch (the re-quantisation scale needs every row), the oracle's e4m3 encoder for the sampled rows, fp32
+    down projection."""
     from dynaflow_amd.backend import make_backend
     from dynaflow_amd.config import CUDAGraphConfig, DynaFlowConfig, InductorConfig
     from dynaflow_amd.fp8_mlp import Fp8SwiGLU
@@ -447,40 +452,63 @@ def test_fp8_config_full_size_properties():
     ws = [(torch.randn(s, generator=gen, device="cuda") * 0.02).bfloat16() for s in ((inter, hidden), (inter, hidden), (hidden, inter))]
     layer = Fp8SwiGLU.from_weights(*ws)
     del ws
-    cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", 4, InductorConfig(enabled=True),
-                         CUDAGraphConfig(enabled=False, capture_sizes=[tokens]),
-                         {"min_nano_split_tokens": 64, "num_nano_batches": 4, "dump_graph": False})
-    manager = DynaFlowManager()
-    torch._dynamo.reset()
-    torch._dynamo.mark_dynamic(x, 0)
-    compiled = torch.compile(layer, backend=make_backend(manager, cfg), fullgraph=True)
-    with torch.no_grad():
-        manager.prepare(tokens, [tokens])
-        compiled(x)
-        split = manager.prepare(tokens, [tokens])
-        y = compiled(x)
-        manager.prepare(tokens, [tokens])
-        y2 = compiled(x)
-        direct = layer.forward_schedule(x, split.split_indices)
-    torch.cuda.synchronize()
-    assert split.split_indices == [0, 2048, 4096, 6144, 8192]
-    assert torch.equal(y, y2) and torch.equal(y, direct)
-    # fp32 evaluation of nano-batch 0, rows 0..7, on the same e4m3 operands
-    from dynaflow_amd import ops
-    xb = x[:2048]
-    xq, xs = ops.quant_fp8(xb)
-    rows = slice(0, 8)
-    xd = xq[rows].float() * xs
-    g = (xd @ (layer.w_gate_q.float() * layer.w_gate_s[:, None]).t()).bfloat16()
-    u = (xd @ (layer.w_up_q.float() * layer.w_up_s[:, None]).t()).bfloat16()
-    # the re-quantisation scale of the SiLU*mul output needs the whole nano-batch: take it from the kernels
-    gate_full = ops.linear_fp8(xq, layer.w_gate_q, xs, layer.w_gate_s)
-    up_full = ops.linear_fp8(xq, layer.w_up_q, xs, layer.w_up_s)
-    aq, a_s = ops.silu_mul_quant_fp8(gate_full, up_full)
-    assert rel_err(gate_full[rows].float(), g.float()) < 2 ** -6
-    assert rel_err(up_full[rows].float(), u.float()) < 2 ** -6
-    want = (aq[rows].float() * a_s) @ (layer.w_down_q.float() * layer.w_down_s[:, None]).t()
-    assert rel_err(y[rows].float(), want) < TOL["fp8"]
+    outputs = {}
+    for fused in (False, True):
+        print(f"config 5 at full size: fused gate/up/SiLU launch = {fused}", flush=True)
+        layer.fuse_gate_up = fused
+        knobs = {"min_nano_split_tokens": 64, "num_nano_batches": 4, "dump_graph": False}
+        if fused:
+            knobs["fuse_silu_epilogue"] = True
+        cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", 4, InductorConfig(enabled=True),
+                             CUDAGraphConfig(enabled=False, capture_sizes=[tokens]), knobs)
+        manager = DynaFlowManager()
+        torch._dynamo.reset()
+        torch._dynamo.mark_dynamic(x, 0)
+        compiled = torch.compile(layer, backend=make_backend(manager, cfg), fullgraph=True)
+        with torch.no_grad():
+            manager.prepare(tokens, [tokens])
+            compiled(x)
+            split = manager.prepare(tokens, [tokens])
+            y = compiled(x)
+            manager.prepare(tokens, [tokens])
+            y2 = compiled(x)
+            direct = layer.forward_schedule(x, split.split_indices)
+        torch.cuda.synchronize()
+        assert split.split_indices == [0, 2048, 4096, 6144, 8192]
+        assert torch.equal(y, y2) and torch.equal(y, direct)
+        if fused:
+            from dynaflow_amd import ops
+            names = [n.target for n in manager.graph_module.graph.nodes if n.op == "call_module"]
+            head = manager.graph_module.__dict__[names[0]].callable_dynamic
+            assert ops.gate_up_silu_quant_fp8 in [n.target for n in head.graph.nodes if n.op == "call_function"]
+        outputs[fused] = y.clone()
+        del manager, compiled, direct, y, y2
+    assert torch.equal(outputs[False], outputs[True])
+
+    fp8_max = 448.0
+    wd = layer.w_down_q.float() * layer.w_down_s[:, None]
+    wg = layer.w_gate_q.float() * layer.w_gate_s[:, None]
+    wu = layer.w_up_q.float() * layer.w_up_s[:, None]
+    for nano_batch, picked in ((0, [0, 1, 777, 2047]), (3, [0, 1024, 2046, 2047])):
+        print(f"config 5 at full size: oracle-side evaluation of nano-batch {nano_batch}", flush=True)
+        xb = x[nano_batch * 2048:(nano_batch + 1) * 2048].float()
+        x_scale = xb.abs().max().clamp_min(1e-12) / fp8_max
+        xd = (xb / x_scale).clamp(-fp8_max, fp8_max).to(torch.float8_e4m3fn).float() * x_scale
+        g = (xd @ wg.t()).bfloat16()
+        u = (xd @ wu.t()).bfloat16()
+        act = mlp.silu_mul_exact(g, u)                       # bf16, whole nano-batch
+        a_scale = act.float().abs().max().clamp_min(1e-12) / fp8_max
+        rows = torch.tensor(picked)
+        scaled = (act[rows.cuda()].float() / a_scale).clamp(-fp8_max, fp8_max).cpu()
+        codes = torch.from_numpy(mlp.e4m3_encode(scaled.numpy()))
+        a_rows = mlp.dequant(codes, a_scale.reshape(1).cpu())
+        want = a_rows.cuda() @ wd.t()
+        got = outputs[True][nano_batch * 2048 + rows.cuda()]
+        err = rel_err(got.float(), want)
+        print(f"config 5 at full size: nano-batch {nano_batch}, sampled rows against the oracle-side evaluation: "
+              f"{err:.4f}", flush=True)
+        assert err < TOL["fp8"]
+        del xb, xd, g, u, act
 
 
 def test_fused_silu_epilogue_schedule():
