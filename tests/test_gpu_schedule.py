@@ -107,9 +107,10 @@ def test_config2_full_size_properties():
 
 
 def test_config2_headline_mode_full_size():
-    """The mode that the bench reports, at full size: SiLU*mul as the epilogue of the gate/up GEMM (one workgroup
-    per compute unit walks four tiles of the 2048-token nano-batch), one stream per nano-batch, the whole schedule
-    as one hipGraph.  (1) sampled rows against the oracle, (2) the same bits as the unfused two-stream schedule,
+    """The mode that the bench reports, at full size: SiLU*mul as the epilogue of the gate/up GEMM, one stream per
+    nano-batch - so the manager plans the kernels for the two launches of a kind that run side by side - and the
+    whole schedule as one hipGraph.  (1) sampled rows against the oracle, (2) the same bits as the unfused schedule
+    with the same stream policy (separate gate, up and SiLU*mul launches; the same plan for the down projection),
     (3) every replay of the graph equals the eager issue, with eager work between the replays."""
     manager, compiled, xg, (x, wg, wu, wd) = build(4096, 4096, 14336, torch.bfloat16, prenorm=True,
                                                    fuse_silu_epilogue=True, whole_graph=True, streams="by_nano_batch")
@@ -119,7 +120,8 @@ def test_config2_headline_mode_full_size():
     rows = torch.tensor([0, 255, 256, 2047, 2048, 3333, 4095])
     want = mlp.mlp_fp32_from(x[rows], wg, wu, wd)
     assert rel_err(eager[rows].float(), want) < TOL["bf16"]
-    plain_manager, plain, xp, _ = build(4096, 4096, 14336, torch.bfloat16, prenorm=True)
+    assert manager.launches_side_by_side(split) == 2
+    plain_manager, plain, xp, _ = build(4096, 4096, 14336, torch.bfloat16, prenorm=True, streams="by_nano_batch")
     unfused, _ = run(plain_manager, plain, xp, 4096)
     assert torch.equal(eager, unfused)
     for _ in range(3):
