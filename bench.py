@@ -70,6 +70,9 @@ def parse_args():
                    help="time the decode-step kernels at the shape of one nano-batch of the decode configuration "
                         "(128 sequences, 32 query / 8 kv heads, 2048 cached positions): RoPE + cache append + "
                         "attention, against the HBM roofline")
+    p.add_argument("--decode-projection-launches", action="store_true",
+                   help="eager launches of the four projections of a decode layer at 128 rows over rotating weight "
+                        "copies (for rocprofv3 counters and kernel traces)")
     p.add_argument("--prefill-attention-kernels", action="store_true",
                    help="time causal prefill attention at the shape of one nano-batch of the decoder-layer "
                         "configuration (4 sequences x 2048 tokens, 32 query / 8 kv heads), PyTorch's fused "
@@ -370,6 +373,36 @@ def decode_projections(torch, ops, iters):
         out[name] = {"one_launch_128_rows_us": replayed(alone), "pair_planned_alone_us": replayed(pairs(1)),
                      "pair_planned_for_two_us": replayed(pairs(2)), "one_launch_256_rows_us": replayed(whole),
                      "weight_bytes": (2 if fused else 1) * n * k * 2}
+        del ws
+    return out
+
+
+def decode_projection_launches(torch, ops, iters):
+    """Eager launches of the four projections of a decode layer at 128 rows, for hardware counters and kernel traces
+    (one kernel per launch, nothing else on the GPU): every projection ``iters`` times over eight rotating weight
+    copies (they come from HBM, as in a 32-layer model), once planned as a lone launch and once with the plan for two
+    launches side by side (the form the two-stream decode schedule runs; traced alone here).  Returns us per launch
+    from HIP events around each loop."""
+    H, I, rows = HIDDEN, INTER, 128
+    gen = torch.Generator(device="cuda").manual_seed(6)
+    out = {}
+    for name, n, k, fused in (("qkv", 6144, H, False), ("o", H, H, False), ("gate_up_silu", I, H, True),
+                              ("down", H, I, False)):
+        x = torch.randn(rows, k, generator=gen, device="cuda").bfloat16()
+        copies = 4 if fused else 8
+        ws = [(torch.randn(n, k, generator=gen, device="cuda") * 0.02).bfloat16() for _ in range(copies)]
+        for share in (1, 2):
+            state = {"i": 0}
+
+            def call():
+                i = state["i"] = (state["i"] + 1) % copies
+                with ops.launch_options(side_by_side=share):
+                    if fused:
+                        ops.gate_up_silu(x, ws[i], ws[(i + 1) % copies])
+                    else:
+                        ops.linear(x, ws[i])
+
+            out[f"{name}_planned_for_{share}_us"] = round(time_kernel(torch, call, iters, warmup=8) * 1e3, 1)
         del ws
     return out
 
@@ -993,6 +1026,9 @@ def main() -> int:
         line = decode_kernels(torch, ops, max(20, args.steps))
         line["projections"] = decode_projections(torch, ops, max(20, args.steps))
         print(json.dumps(line))
+        return 0
+    if args.decode_projection_launches:
+        print(json.dumps(decode_projection_launches(torch, ops, max(16, args.steps))))
         return 0
     if args.prefill_attention_kernels:
         print(json.dumps(prefill_attention_kernels(torch, ops, max(20, args.steps))))

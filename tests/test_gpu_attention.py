@@ -30,7 +30,8 @@ def inputs(B, S, Hq, Hkv, seed):
 
 
 @pytest.mark.parametrize("B,S,Hq,Hkv", [(1, 64, 1, 1), (2, 128, 4, 2), (3, 320, 8, 2), (1, 512, 4, 1), (2, 256, 3, 3),
-                                        (8, 64, 4, 1), (1, 192, 2, 1), (1, 320, 3, 1), (1, 128, 8, 1)])
+                                        (8, 64, 4, 1), (1, 192, 2, 1), (1, 320, 3, 1), (1, 128, 8, 1),
+                                        (2, 448, 16, 4), (1, 1024, 4, 1)])
 def test_causal_attention_against_oracle(ops, B, S, Hq, Hkv):
     q, k, v = inputs(B, S, Hq, Hkv, S + Hq)
     print(f"causal attention B={B} S={S} Hq={Hq} Hkv={Hkv}", flush=True)
@@ -104,12 +105,14 @@ def test_causal_attention_under_graph_capture(ops):
         torch.randn(256, 256, device="cuda").sum().item()
 
 
-def test_causal_attention_scores_that_outgrow_the_first_tile(ops):
+@pytest.mark.parametrize("Hq,Hkv", [(4, 2), (8, 2), (4, 1)])
+def test_causal_attention_scores_that_outgrow_the_first_tile(ops, Hq, Hkv):
     """Rows whose later scores exceed the maximum of their first tile by far more than 2^64: the fast pass
     of those workgroups overflows its sums, notices, and the safe pass recomputes them with a running maximum.
     Half of the (sequence, head) pairs are affected, the others stay on the fast pass; both must match the
-    oracle, and a second call gives the same bits."""
-    B, S, Hq, Hkv = 2, 512, 4, 2
+    oracle, and a second call gives the same bits.  Two and four query heads per kv head: both kernels (64 query
+    rows per wave; 32 rows per wave with two workgroups per compute unit)."""
+    B, S = 2, 512
     q, k, v = inputs(B, S, Hq, Hkv, 77)
     direction = torch.nn.functional.normalize(torch.randn(D, generator=torch.Generator().manual_seed(1)), dim=0)
     q[0] = (q[0].float() + 30.0 * direction).bfloat16()              # sequence 0: queries aligned with ...
