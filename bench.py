@@ -113,8 +113,9 @@ def build_path(torch, x, weights, **knobs):
         model.gate_proj.weight.copy_(wg)
         model.up_proj.weight.copy_(wu)
         model.down_proj.weight.copy_(wd)
-    extra = {"min_nano_split_tokens": 64, "num_nano_batches": SPLITS, "dump_graph": False, **EXTRA_KNOBS}
+    extra = {"min_nano_split_tokens": 64, "num_nano_batches": SPLITS, "dump_graph": False}
     extra.update(knobs)
+    extra.update(EXTRA_KNOBS)          # --knob on the command line wins over the mode's own knobs
     cfg = DynaFlowConfig("dynaflow_amd.schedulers:MLPOverlapScheduler", SPLITS, InductorConfig(enabled=True),
                          CUDAGraphConfig(enabled=False, capture_sizes=[TOKENS]), extra)
     manager = DynaFlowManager()
