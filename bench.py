@@ -61,6 +61,9 @@ def parse_args():
     p.add_argument("--kernels-only", action="store_true",
                    help="run only the single-kernel timing loops plus a 256 MiB device copy (used to calibrate "
                         "FETCH_SIZE / WRITE_SIZE under rocprofv3 --pmc); prints the kernel figures as JSON")
+    p.add_argument("--operands", choices=("random", "zeros"), default="random",
+                   help="with --kernels-only: `zeros` runs the same launches on all-zero operands (no bit toggles in "
+                        "the data paths: what the kernels do when the package power limit is out of the way)")
     p.add_argument("--headline-only", action="store_true",
                    help="only the headline mode (fused epilogue, two streams, one hipGraph): for kernel traces of the step")
     p.add_argument("--fp8", action="store_true",
@@ -1039,6 +1042,10 @@ def main() -> int:
     weights = (wg.cuda(), wu.cuda(), wd.cuda())
 
     if args.kernels_only:
+        if args.operands == "zeros":
+            x.zero_()
+            for w in weights:
+                w.zero_()
         print(json.dumps(single_kernels(torch, ops, x, weights, max(20, args.steps), calibration_copy=True)))
         return 0
 
@@ -1149,6 +1156,13 @@ def main() -> int:
     gemm_flops = 2.0 * mb * HIDDEN * INTER          # one projection of one nano-batch
     silu_bytes = 3.0 * mb * INTER * 2               # read gate + up, write out
     layer_flops = 6.0 * TOKENS * HIDDEN * INTER
+    # the same launches on all-zero operands: the same instructions, memory traffic and stalls, but no bit toggles in
+    # the data paths, so the package stays below its power limit and the clocks stay up
+    x_zero, w_zero = torch.zeros_like(x), tuple(torch.zeros_like(w) for w in weights)
+    kz = single_kernels(torch, ops, x_zero, w_zero, max(20, args.steps))
+    m_z, c_z = build_path(torch, x_zero, w_zero, **HEADLINE_KNOBS)
+    ms_head_zero, _ = time_steps(torch, m_z, c_z, x_zero, args.steps, args.warmup, use_graph=True, settle_s=settle)
+    del m_z, c_z
 
     result = {
         "metric": METRIC,
@@ -1279,6 +1293,21 @@ def main() -> int:
         # 16.8 + 2 x 117.4 MB read, 58.7 MB written
         "traffic": GATE_UP_SILU_SQUARE_TRAFFIC_BYTES,
         "traffic_unit": "bytes per launch",
+    }
+    # how much of the distance to the peak is the package power limit: the same pairs on all-zero operands
+    result["power_limit_check"] = {
+        "what": "the same launches timed the same way on all-zero operands (same instructions, memory traffic and "
+                "stalls; no bit toggles, so the package stays below its 1400 W limit and the clocks stay up)",
+        "gate_up_silu_pair_ms": {"synthetic_operands": ms_gus_pair, "zero_operands": kz["gate_up_silu_pair_ms"]},
+        "down_pair_ms": {"synthetic_operands": ms_down_pair, "zero_operands": kz["down_pair_ms"]},
+        "gate_up_silu_pair_frac_of_peak_on_zero_operands":
+            4 * gemm_flops / (kz["gate_up_silu_pair_ms"] * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
+        "down_pair_frac_of_peak_on_zero_operands":
+            2 * gemm_flops / (kz["down_pair_ms"] * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
+        "rocblas_same_gemm_ms": {"synthetic_operands": ms_blas, "zero_operands": kz["blas_ms"]},
+        # the whole headline step (same issue mode, same graph shape) on a zero input and zero weights
+        "layer_ms_per_step": {"synthetic_operands": ms_head, "zero_operands": ms_head_zero},
+        "layer_frac_of_peak_on_zero_operands": layer_flops / (ms_head_zero * 1e-3) / 1e12 / BF16_MFMA_PEAK_TFLOPS,
     }
     # ---- the same figures under sustained load
     if load_s > 0:
