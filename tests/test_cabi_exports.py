@@ -184,3 +184,24 @@ def test_the_product_never_imports_the_oracle():
                 inside = {id(n) for n in oracle_imports(node)}
         assert inside, f"{name}: {allowed} was expected to use the oracle"
         assert {id(n) for n in oracle_imports(tree)} == inside, f"{name} imports the oracle outside {allowed}"
+
+
+def test_bench_refuses_more_than_one_gpu_and_a_box_without_one():
+    """`bench.py --gpus N` with N above 1 exits with a message that says so (before anything touches a GPU), and
+    on a machine without a GPU the default run says that it needs one instead of printing a figure."""
+    import pathlib
+    import subprocess
+    import sys
+
+    root = pathlib.Path(__file__).resolve().parents[1]
+    many = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                          timeout=120)
+    assert many.returncode != 0 and many.stdout.strip() == ""
+    assert "one GPU" in many.stderr and "--gpus 2" in many.stderr
+    import torch
+
+    if torch.cuda.is_available():
+        return
+    none = subprocess.run([sys.executable, str(root / "bench.py")], capture_output=True, text=True, timeout=300)
+    assert none.returncode != 0 and none.stdout.strip() == ""
+    assert "no GPU" in none.stderr
