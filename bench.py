@@ -158,6 +158,43 @@ def time_steps(torch, manager, compiled, x, steps, warmup, use_graph, settle_s=0
     return (t1 - t0) * 1e3 / steps, y
 
 
+def vendor_library_layer(torch, x, weights, steps, warmup, settle_s):
+    """ms per step of ``down(silu(gate(x)) * up(x))`` on the whole batch through ``torch.nn.functional`` (the vendor's
+    GEMM library, aten's SiLU and multiplication), captured once and replayed as one graph; timed like every other
+    loop of this file.  A yardstick, not part of the path."""
+    import torch.nn.functional as F
+
+    wg, wu, wd = weights
+    side = torch.cuda.Stream()
+    with torch.no_grad():
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                F.linear(F.silu(F.linear(x, wg)) * F.linear(x, wu), wd)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y = F.linear(F.silu(F.linear(x, wg)) * F.linear(x, wu), wd)
+        torch.cuda.synchronize()
+        if settle_s > 0:
+            until = time.perf_counter() + settle_s
+            while time.perf_counter() < until:
+                for _ in range(10):
+                    graph.replay()
+                torch.cuda.synchronize()
+        for _ in range(warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    del graph, y
+    return (t1 - t0) * 1e3 / steps
+
+
 def gpu_time_of_steps(torch, manager, compiled, x, steps):
     """GPU-side duration of one eagerly issued step (median over ``steps``, ms): the GPU is kept busy with a
     spin kernel while the host issues the whole step behind it, so the interval between the two events holds the
@@ -1135,6 +1172,9 @@ def main() -> int:
     # ---- for comparison only: the 4096 tokens as ONE batch (no nano-batches, one stream, two launches)
     m_un, c_un = build_path(torch, x, weights, min_nano_split_tokens=1 << 30, fuse_silu_epilogue=True)
     ms_unsplit_gpu = gpu_time_of_steps(torch, m_un, c_un, x, min(args.steps, 20))
+    # for scale: the same layer on the whole batch through PyTorch's own operators (the vendor GEMM library and aten's
+    # SiLU and multiplication), replayed as one graph on one stream so that no host time is in the figure
+    ms_vendor = vendor_library_layer(torch, x, weights, args.steps, args.warmup, settle)
 
     if not (head_identical and fused_identical and identical and serial_graph_identical and pair_identical):
         print("bench.py: issue modes that run the same kernels disagree bit for bit: "
@@ -1211,7 +1251,9 @@ def main() -> int:
         },
         # reported beside the nano-batch schedule, never as `value`: every operator of this layer is MFMA-bound, so
         # on one GPU two nano-batches have nothing of a different kind to hide behind each other
-        "unsplit_one_batch": {"silu_mul_as_gemm_epilogue_gpu_side_ms": ms_unsplit_gpu},
+        "unsplit_one_batch": {"silu_mul_as_gemm_epilogue_gpu_side_ms": ms_unsplit_gpu,
+                              "pytorch_operators_one_graph_ms": ms_vendor,
+                              "headline_over_pytorch_operators": ms_vendor / ms_head},
         "overlap": {
             "serialized_ms": ms_serial,
             "serialized_gpu_side_ms": ms_serial_gpu,
