@@ -20,10 +20,11 @@
 //     on the global side by choosing which chunk each lane fetches.  Fragment reads
 //     (ds_read_b128, row = lane%32, chunk = 2*ks + lane/32) are then conflict free.
 //   * one wave per SIMD means nothing hides a stall, so the loop body is pinned
-//     instruction by instruction: after every MFMA at most one LDS read or one DMA
-//     issue, fragments of k-step s+1 are read while step s multiplies, and the
-//     workgroup barrier that hands LDS units back sits between k-steps 2 and 3 with
-//     MFMAs already in the pipe.
+//     instruction by instruction: the two k-steps of a slab go into one accumulator
+//     block as a pair of MFMAs (the second adds to what the first has just written),
+//     behind a pair comes at most one LDS read or one DMA issue, fragments are read
+//     into registers that the walk over the 8 x 8 blocks has just freed, and the
+//     workgroup barrier that hands LDS units back sits in the middle of a slab.
 //   * the loop is branch free: halves past the end of K re-read the last slab into
 //     units nobody reads, so the count of outstanding DMA instructions is the same in
 //     every iteration (s_waitcnt vmcnt(8) before the barrier).
@@ -263,6 +264,14 @@ DFHIP_DEVICE int fused_pair_output_of(int pos) {
   return 32 * (j >> 1) + 8 * (n >> 2) + 4 * (j & 1) + (n & 3);
 }
 
+template <int I, int N, class F>
+DFHIP_DEVICE void static_for(F& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
 // FUSED = false: C[M,N] = A W^T.
 // FUSED = true : C[M,N] = silu(A W^T) * (A W2^T) with W = gate weight, W2 = up weight, N = the
 //   intermediate size.  A tile is 256 rows x 128 columns; its "W half" holds 128 gate rows and 128 up
@@ -272,7 +281,10 @@ DFHIP_DEVICE int fused_pair_output_of(int pos) {
 // The products are v_mfma_f32_16x16x32_bf16: a wave's 128 x 128 block is 8 x 8 blocks of 16 x 16, a slab
 // of 64 is two k-steps of 32.  Per flop the instruction reads half as many accumulator registers as the
 // 32x32x16 one; a loop of nothing but this instruction sustains about 15 % more at the package power
-// limit, and this kernel ran 9-10 % faster than its 32x32x16 predecessor with the same ring.
+// limit, and this kernel ran 9-10 % faster than its 32x32x16 predecessor with the same ring.  The two
+// k-steps of a slab go into a block as one pair of instructions: the second takes the accumulator straight
+// from the first (a loop of nothing but such pairs sustains another 6 % at the power limit; this kernel gained
+// 1.3 % over walking all 64 blocks per k-step, after paying 1.8 % more cycles for the order of its reads).
 //   fragment of a 16-row block for k-step ks: lane -> row lane%16, 16-byte chunk 4*ks + lane/16
 //   acc[i][j] (W block j first operand, A block i second): lane holds
 //     C[16 i + lane%16][16 j + 4 (lane/16) + r], r = 0..3
@@ -350,34 +362,68 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
   wait_vmcnt<16>();   // slab 0 has landed; slab 1 may still be in flight
   workgroup_barrier();
 
-  bf16x8 fa[2][8], fw[2][8];
-  // fragments in the order the MFMAs need them: W block 0, A block 0, W blocks 1..7, A blocks 1..7
-  auto read_frag = [&](int pos, int ks, int slot, int unit_a, int unit_w) {
-    const bool is_a = pos == 1 || pos > 8;
-    const int blk = pos == 0 ? 0 : pos == 1 ? 0 : pos <= 8 ? pos - 1 : pos - 8;
-    if (is_a)
-      fa[slot][blk] = *reinterpret_cast<const bf16x8*>(smem + unit_a * UNIT + a_lane + koff[ks] + blk * 2048);
+  // K loop.  The two k-steps of a slab go into one 16 x 16 block back to back: the second product adds to the
+  // accumulator that the first one has just written, which the matrix pipe hands over without the round trip
+  // through the register file - less energy per product, and energy is what bounds this kernel.  For that, the W
+  // fragments of a slab (both k-steps, 16 fragments) are in registers before its first product, and the 8 x 8
+  // blocks are walked so that registers free up on the way:
+  //   top half    rows 0 .. 3, row by row; behind the pairs of row i, the A fragments of row i + 1 and of row
+  //               4 + i (and, in row 0, the W fragments of column 7, whose registers the last slab used to its end);
+  //   bottom half rows 4 .. 7, column by column; behind column j its W fragments are dead and the registers
+  //               take those of the next slab, which row 0 needs first.
+  // A pair is one statement (nothing between its two instructions); behind a pair comes at most one LDS read
+  // or one DMA issue.
+  bf16x8 fa_top[2][2], fa_bot[4][2], fw[2][8];   // [row parity][k-step], [row - 4][k-step], [k-step][block]
+  auto a_frag = [&](int row, int ks, int unit) {
+    return *reinterpret_cast<const bf16x8*>(smem + unit * UNIT + a_lane + koff[ks] + row * 2048);
+  };
+  auto read_w = [&](int blk, int ks, int unit) {
+    fw[ks][blk] = *reinterpret_cast<const bf16x8*>(smem + unit * UNIT + w_lane + koff[ks] + blk * 2048);
+  };
+  // written out so that the accumulator stays in its own registers (the compiler otherwise gives result and
+  // addend different registers and moves 64 accumulators around in every iteration)
+  auto mfma_pair = [&](int i, int j) {
+    if (i < 4)
+      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\tv_mfma_f32_16x16x32_bf16 %0, %3, %4, %0"
+                   : "+a"(acc[i][j])
+                   : "v"(fw[0][j]), "v"(fa_top[i & 1][0]), "v"(fw[1][j]), "v"(fa_top[i & 1][1]));
     else
-      fw[slot][blk] = *reinterpret_cast<const bf16x8*>(smem + unit_w * UNIT + w_lane + koff[ks] + blk * 2048);
+      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\tv_mfma_f32_16x16x32_bf16 %0, %3, %4, %0"
+                   : "+a"(acc[i][j])
+                   : "v"(fw[0][j]), "v"(fa_bot[i - 4][0]), "v"(fw[1][j]), "v"(fa_bot[i - 4][1]));
   };
-  auto mfma = [&](int q, int slot) {   // snake over the 8 x 8 blocks: one operand changes per instruction
-    const int i = q >> 3, j = (i & 1) ? 7 - (q & 7) : (q & 7);
-    // written out so that the accumulator stays in its own registers (the compiler otherwise gives result and
-    // addend different registers and moves 64 accumulators around in every iteration)
-    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fw[slot][j]), "v"(fa[slot][i]));
-  };
+  // the zeros are in the accumulators before the first product reads them (the compiler would otherwise move
+  // them in right in front of it, and does not know the wait states that a product needs after such a move)
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
+  asm volatile("s_nop 7" ::: "memory");
 
   int ua = 0, uw = 1;   // units of the slab being multiplied
   int ia = 4, iw = 0;   // units that A(kt+2) and W(kt+2) go to
 #pragma unroll
-  for (int pos = 0; pos < 16; ++pos) read_frag(pos, 0, 0, ua, uw);
-  for (int kt = 0; kt < KT; ++kt) {
-    // k-step 0: the fragments of k-step 1 behind MFMAs 0..15, the DMA of A(kt+2) behind every sixth after that
+  for (int j = 0; j < 8; ++j) { read_w(j, 0, uw); read_w(j, 1, uw); }
+  fa_top[0][0] = a_frag(0, 0, ua);
+  fa_top[0][1] = a_frag(0, 1, ua);
+  // all of them have landed before the loop: the loop's first wait then has to cover what an iteration leaves
+  // in flight (the refills of the last columns), not the order of the reads above
 #pragma unroll
-    for (int q = 0; q < 64; ++q) {
-      mfma(q, 0);
-      if (q < 16) read_frag(q, 1, 1, ua, uw);
-      else if ((q - 16) % 6 == 0) dma_a((q - 16) / 6, kt + 2, ia);
+  for (int j = 0; j < 8; ++j) asm volatile("" ::"v"(fw[0][j]), "v"(fw[1][j]));
+  asm volatile("" ::"v"(fa_top[0][0]), "v"(fa_top[0][1]));
+  for (int kt = 0; kt < KT; ++kt) {
+    // top half.  Behind pair j of row i: row 0 starts with the two W fragments of column 7 (from this slab's unit:
+    // at kt = 0 that reads again what is there); then the two A fragments of row i + 1, the two of row 4 + i; in
+    // rows 1 .. 3 the DMA of A(kt+2) behind the last three pairs
+#pragma unroll
+    for (int p = 0; p < 32; ++p) {
+      const int i = p >> 3, j = p & 7;
+      mfma_pair(i, j);
+      const int first = i == 0 ? 2 : 0;
+      if (i == 0 && j < 2) read_w(7, j, uw);
+      else if (j - first < 2) { if (i < 3) fa_top[(i + 1) & 1][j - first] = a_frag(i + 1, j - first, ua); }
+      else if (j - first < 4) fa_bot[i][j - first - 2] = a_frag(4 + i, j - first - 2, ua);
+      else if (i >= 1 && j >= 5) { if ((i - 1) * 3 + j - 5 < 8) dma_a((i - 1) * 3 + j - 5, kt + 2, ia); }
       DFHIP_PIN;
     }
     // every LDS read of slab kt has been issued; once they have landed its two units are free.
@@ -387,13 +433,19 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
     workgroup_barrier();
     int na = ua + 2; if (na >= NUNITS) na -= NUNITS;
     int nw = uw + 2; if (nw >= NUNITS) nw -= NUNITS;
-    // k-step 1: the DMA of W(kt+2) into the unit A(kt) just left behind every fourth MFMA, then the
-    // fragments of slab kt+1, k-step 0
+    // bottom half.  Column j is four pairs: behind the second and third, the W fragments of slab kt+1 for column
+    // j - 1 (column 0: its A fragments of row 0); behind the first and last of columns 0 .. 3, the DMA of
+    // W(kt+2) into the unit A(kt) just left
 #pragma unroll
-    for (int q = 0; q < 64; ++q) {
-      mfma(q, 1);
-      if (q < 32) { if (q % 4 == 0) dma_w(q / 4, kt + 2, iw); }
-      else if (q < 48) read_frag(q - 32, 0, 0, na, nw);
+    for (int p = 0; p < 32; ++p) {
+      const int j = p >> 2, r = p & 3, i = 4 + r;
+      mfma_pair(i, j);
+      if (r == 1 || r == 2) {
+        if (j == 0) fa_top[0][r - 1] = a_frag(0, r - 1, na);
+        else read_w(j - 1, r - 1, nw);
+      } else if (j < 4) {
+        dma_w(j * 2 + (r == 3), kt + 2, iw);
+      }
       DFHIP_PIN;
     }
     ua = na; uw = nw;
@@ -796,14 +848,6 @@ int launch_ring224(const void* A, int64_t lda, const void* W, const void* W2, in
 constexpr int WALK_STORES = WALK_STORES_PER_SLAB;    // stores behind one slab of the next tile
 constexpr int WALK_PEEL = 16 / WALK_STORES;          // iterations of the next tile that carry stores
 constexpr int WALK_MIN_SLABS = WALK_PEEL + 3;
-
-template <int I, int N, class F>
-DFHIP_DEVICE void static_for(F& f) {
-  if constexpr (I < N) {
-    f(std::integral_constant<int, I>{});
-    static_for<I + 1, N>(f);
-  }
-}
 
 __global__ void __launch_bounds__(RTHREADS)
 gemm_bf16_gate_up_silu_walk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
