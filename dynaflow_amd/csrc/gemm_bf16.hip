@@ -392,6 +392,26 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
                    : "+a"(acc[i][j])
                    : "v"(fw[0][j]), "v"(fa_bot[i - 4][0]), "v"(fw[1][j]), "v"(fa_bot[i - 4][1]));
   };
+  // a pair with one DMA instruction behind it, as one statement: m0 is set ahead of the pair (which also is the
+  // wait state that the DMA instruction needs after the move), so that only the DMA instruction itself stands
+  // between this pair and the next
+  auto mfma_pair_dma = [&](int i, int j, uint32_t lds_addr, const void* base, uint32_t offset) {
+    if (i < 4)
+      asm volatile("s_mov_b32 m0, %5\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\tv_mfma_f32_16x16x32_bf16 %0, %3, %4, %0"
+                   "\n\tglobal_load_lds_dwordx4 %6, %7"
+                   : "+a"(acc[i][j])
+                   : "v"(fw[0][j]), "v"(fa_top[i & 1][0]), "v"(fw[1][j]), "v"(fa_top[i & 1][1]), "s"(lds_addr),
+                     "v"(offset), "s"(base)
+                   : "memory", "m0");
+    else
+      asm volatile("s_mov_b32 m0, %5\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\tv_mfma_f32_16x16x32_bf16 %0, %3, %4, %0"
+                   "\n\tglobal_load_lds_dwordx4 %6, %7"
+                   : "+a"(acc[i][j])
+                   : "v"(fw[0][j]), "v"(fa_bot[i - 4][0]), "v"(fw[1][j]), "v"(fa_bot[i - 4][1]), "s"(lds_addr),
+                     "v"(offset), "s"(base)
+                   : "memory", "m0");
+  };
+  auto slab_of = [&](int slab) { return slab0 + (slab < KT ? slab : KT - 1); };
   // the zeros are in the accumulators before the first product reads them (the compiler would otherwise move
   // them in right in front of it, and does not know the wait states that a product needs after such a move)
 #pragma unroll
@@ -418,12 +438,16 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
 #pragma unroll
     for (int p = 0; p < 32; ++p) {
       const int i = p >> 3, j = p & 7;
-      mfma_pair(i, j);
       const int first = i == 0 ? 2 : 0;
-      if (i == 0 && j < 2) read_w(7, j, uw);
-      else if (j - first < 2) { if (i < 3) fa_top[(i + 1) & 1][j - first] = a_frag(i + 1, j - first, ua); }
-      else if (j - first < 4) fa_bot[i][j - first - 2] = a_frag(4 + i, j - first - 2, ua);
-      else if (i >= 1 && j >= 5) { if ((i - 1) * 3 + j - 5 < 8) dma_a((i - 1) * 3 + j - 5, kt + 2, ia); }
+      const int t = (i - 1) * 3 + j - 5;               // DMA instruction of A(kt+2) behind this pair, if any
+      if (i >= 1 && j >= 5 && t < 8) {
+        mfma_pair_dma(i, j, ia * UNIT + wave_lds + t * 1024, a_tile + (int64_t)slab_of(kt + 2) * (BK * 2), a_off[t]);
+      } else {
+        mfma_pair(i, j);
+        if (i == 0 && j < 2) read_w(7, j, uw);
+        else if (j - first < 2) { if (i < 3) fa_top[(i + 1) & 1][j - first] = a_frag(i + 1, j - first, ua); }
+        else if (j - first < 4) fa_bot[i][j - first - 2] = a_frag(4 + i, j - first - 2, ua);
+      }
       DFHIP_PIN;
     }
     // every LDS read of slab kt has been issued; once they have landed its two units are free.
@@ -439,12 +463,15 @@ gemm_bf16_ring_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict
 #pragma unroll
     for (int p = 0; p < 32; ++p) {
       const int j = p >> 2, r = p & 3, i = 4 + r;
-      mfma_pair(i, j);
       if (r == 1 || r == 2) {
+        mfma_pair(i, j);
         if (j == 0) fa_top[0][r - 1] = a_frag(0, r - 1, na);
         else read_w(j - 1, r - 1, nw);
       } else if (j < 4) {
-        dma_w(j * 2 + (r == 3), kt + 2, iw);
+        const int t = j * 2 + (r == 3);
+        mfma_pair_dma(i, j, iw * UNIT + wave_lds + t * 1024, w_tile + (int64_t)slab_of(kt + 2) * (BK * 2), w_off[t]);
+      } else {
+        mfma_pair(i, j);
       }
       DFHIP_PIN;
     }
